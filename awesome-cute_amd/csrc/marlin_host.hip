@@ -1,0 +1,257 @@
+// Host launcher and C ABI of the gfx950 W4A16 Marlin GEMM.
+//
+// Mirrors the host side of the reference path: the argument contract and
+// shape checks of marlin_cute (marlin_cute_kernel.cu:28-115) and the checks
+// of the tensor binding mul (marlin_gemm.cpp:19-56).  Kernel choice, grid and
+// partition are this library's own.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "../../include/marlin_amd.h"
+#include "w4a16_common.hpp"
+
+namespace {
+
+using namespace w4a16;
+
+constexpr int kMaxStreamGrid = 1024;  // workgroups of the streaming kernel
+constexpr int kMaxDevices = 16;
+
+thread_local char g_last_error[256] = "";
+
+void set_error(hipError_t e, const char* what) {
+  snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
+}
+
+// Partial-sum scratch of the streaming kernel: one buffer per (device, stream)
+// so that GEMMs on different streams never share partial sums.  Buffers live
+// until the process ends.
+struct Scratch {
+  hipStream_t stream;
+  float* ptr;
+};
+struct DeviceState {
+  int cus = 0;
+  std::vector<Scratch> scratch;
+};
+std::mutex g_mu;
+DeviceState g_dev[kMaxDevices];
+
+constexpr size_t kScratchBytes = (size_t)2 * kMaxStreamGrid * stream_slot_bytes(4);
+
+int device_cus(int dev) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_dev[dev].cus == 0) {
+    int cus = 0;
+    hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) {
+      set_error(e, "hipDeviceGetAttribute");
+      return -1;
+    }
+    g_dev[dev].cus = cus;
+  }
+  return g_dev[dev].cus;
+}
+
+float* scratch_for(int dev, hipStream_t stream) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  for (const Scratch& s : g_dev[dev].scratch)
+    if (s.stream == stream) return s.ptr;
+  float* p = nullptr;
+  hipError_t e = hipMalloc((void**)&p, kScratchBytes);
+  if (e != hipSuccess) {
+    set_error(e, "hipMalloc(scratch)");
+    return nullptr;
+  }
+  g_dev[dev].scratch.push_back({stream, p});
+  return p;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
+
+// Shape checks in the order the reference performs them
+// (marlin_cute_kernel.cu:39-60, 95-107).
+int check_shape(int m, int n, int k, int groupsize, int& thread_k, int& thread_n) {
+  if (thread_k == -1 || thread_n == -1) {
+    if (m <= 16) {
+      thread_k = 128;
+      thread_n = 128;
+    } else {
+      thread_k = 64;
+      thread_n = 256;
+    }
+  }
+  if (thread_k <= 0 || thread_n <= 0) return MARLIN_ERR_PROB_SHAPE;
+  if (groupsize == 0 || groupsize < -1) return MARLIN_ERR_KERN_SHAPE;
+  const int group_blocks = groupsize == -1 ? -1 : groupsize / 16;
+  if (group_blocks == 0) return MARLIN_ERR_KERN_SHAPE;
+  if (m < 0 || n < 0 || k < 0) return MARLIN_ERR_PROB_SHAPE;
+  if (n % thread_n != 0 || k % thread_k != 0 || (group_blocks != -1 && k % group_blocks != 0))
+    return MARLIN_ERR_PROB_SHAPE;
+  if (m == 0 || n == 0 || k == 0) return MARLIN_OK;
+  // kernel table: tiles (128 k x 128 n) for one 16-row block, (64 k x 256 n)
+  // for one to four; group size 128 or per-channel
+  if (groupsize != -1 && groupsize != 128) return MARLIN_ERR_KERN_SHAPE;
+  const bool small = thread_k == 128 && thread_n == 128;
+  const bool wide = thread_k == 64 && thread_n == 256;
+  if (!small && !wide) return MARLIN_ERR_KERN_SHAPE;
+  if (small && m > 16) return MARLIN_ERR_KERN_SHAPE;
+  if (groupsize == 128 && k % 128 != 0) return MARLIN_ERR_PROB_SHAPE;
+  return MARLIN_OK;
+}
+
+struct Plan {
+  int kernel;  // 1 streaming, 2 prefill
+  int grid;
+  StreamPlan sp;
+  int launches;
+};
+
+constexpr int kStreamMaxRows = 64;
+
+Plan make_plan(int m, int n, int k, int sms, int cus) {
+  Plan pl;
+  pl.kernel = 1;
+  int want = sms > 0 ? sms : cus * env_int("MARLIN_AMD_STREAM_WG_PER_CU", 1);
+  if (want > kMaxStreamGrid) want = kMaxStreamGrid;
+  pl.sp = make_stream_plan(n, k, want);
+  pl.grid = pl.sp.grid;
+  pl.launches = ceil_div(m, kStreamMaxRows);
+  return pl;
+}
+
+int run(const void* A, const void* B, void* C, const void* s, int m, int n, int k,
+        void* workspace, int groupsize, int dev, hipStream_t stream, int thread_k, int thread_n,
+        int sms) {
+  int rc = check_shape(m, n, k, groupsize, thread_k, thread_n);
+  if (rc != MARLIN_OK || m == 0 || n == 0 || k == 0) return rc;
+  if (dev < 0 || dev >= kMaxDevices) {
+    snprintf(g_last_error, sizeof(g_last_error), "device index %d out of range", dev);
+    return MARLIN_ERR_RUNTIME;
+  }
+  int prev = -1;
+  hipError_t e = hipGetDevice(&prev);
+  if (e != hipSuccess) {
+    set_error(e, "hipGetDevice");
+    return MARLIN_ERR_RUNTIME;
+  }
+  if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) {
+    set_error(e, "hipSetDevice");
+    return MARLIN_ERR_RUNTIME;
+  }
+  int cus = device_cus(dev);
+  rc = MARLIN_ERR_RUNTIME;
+  if (cus > 0) {
+    Plan pl = make_plan(m, n, k, sms, cus);
+    float* scratch = scratch_for(dev, stream);
+    if (scratch) {
+      rc = MARLIN_OK;
+      for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
+        GemmArgs a;
+        a.A = (const char*)A + (size_t)m0 * k * 2;
+        a.B = B;
+        a.C = (char*)C + (size_t)m0 * n * 2;
+        a.S = s;
+        a.M = m - m0 < kStreamMaxRows ? m - m0 : kStreamMaxRows;
+        a.N = n;
+        a.K = k;
+        a.locks = (int*)workspace;
+        a.scratch = scratch;
+        a.gpb = pl.sp.gpb;
+        rc = launch_stream(a, groupsize != -1, pl.grid, stream);
+      }
+      if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
+    }
+  }
+  if (prev != dev) (void)hipSetDevice(prev);
+  return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+int marlin_gemm(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n,
+                int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k,
+                int thread_n, int sms, int max_par) {
+  (void)max_par;
+  return run(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, (hipStream_t)stream,
+             thread_k, thread_n, sms);
+}
+
+int marlin_cute(const void* A, const void* B, void* C, void* s, int prob_m, int prob_n,
+                int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k,
+                int thread_n, int sms, int max_par) {
+  return marlin_gemm(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream,
+                     thread_k, thread_n, sms, max_par);
+}
+
+int marlin_official(const void* A, const void* B, void* C, void* s, int prob_m, int prob_n,
+                    int prob_k, void* workspace, int groupsize, int dev, void* stream,
+                    int thread_k, int thread_n, int sms, int max_par) {
+  return marlin_gemm(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream,
+                     thread_k, thread_n, sms, max_par);
+}
+
+int marlin_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n,
+               int prob_k, int s_rows, void* workspace, long long workspace_numel, int dev,
+               void* stream, int thread_k, int thread_n, int sms, int max_par, int cute_version,
+               char* err, int err_len) {
+  (void)cute_version;  // one implementation serves both reference variants
+  auto fail = [&](int code, const char* fmt, auto... args) {
+    if (err && err_len > 0) snprintf(err, (size_t)err_len, fmt, args...);
+    return code;
+  };
+  if (err && err_len > 0) err[0] = 0;
+  if (s_rows <= 0) return fail(MARLIN_ERR_GROUPS, "k=%d not compatible with %d groups.", prob_k, s_rows);
+  int groupsize = s_rows == 1 ? -1 : prob_k / s_rows;
+  if (groupsize != -1 && groupsize * s_rows != prob_k)
+    return fail(MARLIN_ERR_GROUPS, "k=%d not compatible with %d groups.", prob_k, s_rows);
+  if (workspace_numel < (long long)(prob_n / 128) * max_par)
+    return fail(MARLIN_ERR_WORKSPACE, "workspace must be of size at least %d.",
+                prob_n / 128 * max_par);
+  int rc = marlin_gemm(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream,
+                       thread_k, thread_n, sms, max_par);
+  if (rc == MARLIN_ERR_PROB_SHAPE)
+    return fail(rc, "Problem (m=%d, n=%d, k=%d) not compatible with thread_k=%d, thread_n=%d.",
+                prob_m, prob_n, prob_k, thread_k, thread_n);
+  if (rc == MARLIN_ERR_KERN_SHAPE)
+    return fail(rc, "No kernel implementation for thread_k=%d, thread_n=%d, groupsize=%d.",
+                thread_k, thread_n, groupsize);
+  if (rc == MARLIN_ERR_RUNTIME) return fail(rc, "HIP runtime error: %s", g_last_error);
+  return rc;
+}
+
+int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                     int thread_n) {
+  return check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
+}
+
+int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                    int thread_n, int sms, int cus, int* out) {
+  for (int i = 0; i < 6; i++) out[i] = 0;
+  int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
+  if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
+  Plan pl = make_plan(prob_m, prob_n, prob_k, sms, cus);
+  out[0] = pl.kernel;
+  out[1] = pl.grid;
+  out[2] = pl.sp.gpb;
+  out[3] = pl.sp.NT;
+  out[4] = pl.sp.KG;
+  out[5] = pl.launches;
+  return rc;
+}
+
+const char* marlin_amd_last_error(void) { return g_last_error; }
+
+const char* marlin_amd_version(void) { return "marlin_amd 0.1 (gfx950)"; }
+
+}  // extern "C"

@@ -1,0 +1,201 @@
+"""Host-side mirror of the reference's `marlin` module (gemm/marlin_gemm/marlin.py)
+over the C ABI of libmarlin_amd.so: `mul`, `Layer`, `replace_linear`, and the
+packing permutations.  The GEMM itself always runs in the HIP library; there is
+no fallback path, and a missing library is an import-time error.
+"""
+import ctypes
+import os
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmarlin_amd.so")
+
+if not os.path.exists(_LIB_PATH):
+    raise ImportError(
+        f"{_LIB_PATH} is missing: build it first (python __graft_entry__.py build, or "
+        "python awesome-cute_amd/build.py); the W4A16 GEMM has no other implementation")
+_lib = ctypes.CDLL(_LIB_PATH)
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_lib.marlin_mul.restype = _I
+_lib.marlin_mul.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P, ctypes.c_longlong, _I, _P,
+                            _I, _I, _I, _I, _I, ctypes.c_char_p, _I]
+_lib.marlin_gemm.restype = _I
+_lib.marlin_gemm.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I]
+_lib.marlin_amd_check.restype = _I
+_lib.marlin_amd_check.argtypes = [_I] * 6
+_lib.marlin_amd_plan.restype = _I
+_lib.marlin_amd_plan.argtypes = [_I] * 8 + [_P]
+_lib.marlin_amd_last_error.restype = ctypes.c_char_p
+_lib.marlin_amd_version.restype = ctypes.c_char_p
+
+
+def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16, cute_version=True):
+    """FP16 x INT4 multiply, C = A @ dequant(B); interface of reference marlin.py:11-24.
+
+    A: (m, k) half, row-major.  B: (k/16, 2n) int32 in Marlin format (`Layer.pack`).
+    C: (m, n) half, overwritten.  s: (k/groupsize, n) half scales, or (1, n).
+    workspace: at least n/128*max_par zero int32 entries; zero again afterwards.
+    thread_k / thread_n / sms: tile and grid hints, -1 = automatic.
+    cute_version: accepted for compatibility; both values run the same kernels.
+    Asynchronous on the current stream of A's device.  Raises RuntimeError where
+    the reference binding raises (marlin_gemm.cpp:27-31,48-55).
+    """
+    for name, t in (("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)):
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a GPU tensor")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    dev = A.get_device()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    err = ctypes.create_string_buffer(512)
+    rc = _lib.marlin_mul(A.data_ptr(), B.data_ptr(), C.data_ptr(), s.data_ptr(),
+                         A.size(0), C.size(1), A.size(1), s.size(0),
+                         workspace.data_ptr(), workspace.numel(), dev, stream,
+                         thread_k, thread_n, sms, max_par, int(bool(cute_version)),
+                         err, len(err))
+    if rc != 0:
+        raise RuntimeError(err.value.decode() or f"marlin_mul failed with code {rc}")
+
+
+# ---------------------------------------------------------------------------
+# Packed layout.  Word w (0..127) of a 16 x 64 block belongs to Marlin lane
+# w // 4 = 4c + t and 16-column tile j = w % 4; its nibble e holds
+# k = 2t + (e >> 2 & 1) + 8 (e & 1),  n = 16 j + c + 8 (e >> 1 & 1).
+
+def _block_coords():
+    w = np.arange(128)[:, None]
+    e = np.arange(8)[None, :]
+    lane, j = w // 4, w % 4
+    t, c = lane % 4, lane // 4
+    k = 2 * t + ((e >> 2) & 1) + 8 * (e & 1)
+    n = 16 * j + c + 8 * ((e >> 1) & 1)
+    return k, n
+
+
+def _get_perms():
+    """Same three permutations as reference marlin.py:29-55, from the closed form:
+    `perm` gathers a run of four row-major 16x16 tiles into nibble order."""
+    k, n = _block_coords()
+    perm = (256 * (n // 16) + 16 * k + n % 16).reshape(-1)
+    scale_perm = [i + 8 * j for i in range(8) for j in range(8)]
+    scale_perm_single = [2 * i + o for i in range(4) for o in (0, 1, 8, 9, 16, 17, 24, 25)]
+    return torch.from_numpy(perm.astype(np.int64)), scale_perm, scale_perm_single
+
+
+_perm, _scale_perm, _scale_perm_single = _get_perms()
+_k_in_block, _n_in_block = _block_coords()
+_block_gather = torch.from_numpy((64 * _k_in_block + _n_in_block).reshape(-1).astype(np.int64))
+
+
+def pack_weights(q):
+    """(k, n) integer tensor with values in [0, 15] -> (k/16, 2n) int32 Marlin words."""
+    k, n = q.shape
+    if k % 16 or n % 64:
+        raise ValueError("k must be divisible by 16 and n by 64")
+    blocks = q.reshape(k // 16, 16, n // 64, 64).permute(0, 2, 1, 3).reshape(k // 16, n // 64, 1024)
+    nib = blocks[:, :, _block_gather.to(q.device)].reshape(k // 16, n // 64, 128, 8).to(torch.int64)
+    shifts = torch.arange(0, 32, 4, device=q.device, dtype=torch.int64)
+    words = (nib << shifts).sum(-1)  # < 2^32
+    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words)
+    return words.reshape(k // 16, 2 * n).to(torch.int32)
+
+
+def pack_scales(s, groupwise):
+    """(groups, n) scales -> the order the kernels read them in (marlin.py:111-118)."""
+    n = s.shape[1]
+    if groupwise:
+        out = s.reshape(-1, 64)[:, _scale_perm]
+    else:
+        out = s.reshape(-1, 32)[:, _scale_perm_single]
+    return out.reshape(-1, n).contiguous()
+
+
+def quantize(w, groupsize=-1):
+    """Symmetric 4-bit quantisation of a (k, n) half weight, as the reference
+    test helper gen_quant4 (marlin_test.py:18-40): per group and column
+    s = max|w| * 2/15, q = clamp(round(w/s) + 8, 0, 15).  Returns the
+    fake-quantised weight (k, n), q (k, n) int32 and s (groups, n)."""
+    k, n = w.shape
+    gs = k if groupsize == -1 else groupsize
+    wg = w.reshape(k // gs, gs, n)
+    s = wg.abs().amax(dim=1, keepdim=True)
+    s = s * (2 / 15)
+    q = torch.clamp(torch.round(wg / s).int() + 8, 0, 15)
+    ref = (q - 8).to(w.dtype) * s
+    return ref.reshape(k, n), q.reshape(k, n), s.reshape(k // gs, n)
+
+
+class Layer(nn.Module):
+    """4-bit (symmetric, grouped) linear layer without bias; interface of reference
+    marlin.py:60-131."""
+
+    def __init__(self, infeatures, outfeatures, groupsize=-1, cute_version=True):
+        super().__init__()
+        if groupsize not in [-1, 128]:
+            raise ValueError('Only groupsize -1 and 128 are supported.')
+        if infeatures % 128 != 0 or outfeatures % 256 != 0:
+            raise ValueError('`infeatures` must be divisible by 128 and `outfeatures` by 256.')
+        if groupsize == -1:
+            groupsize = infeatures
+        if infeatures % groupsize != 0:
+            raise ValueError('`infeatures` must be divisible by `groupsize`.')
+        self.k = infeatures
+        self.n = outfeatures
+        self.groupsize = groupsize
+        self.cute_version = cute_version
+        self.register_buffer('B', torch.empty((self.k // 16, self.n * 16 // 8), dtype=torch.int))
+        self.register_buffer('s', torch.empty((self.k // groupsize, self.n), dtype=torch.half))
+        # sized for the narrowest column tile (128) and the default max_par (16)
+        self.register_buffer('workspace', torch.zeros(self.n // 128 * 16, dtype=torch.int),
+                             persistent=False)
+
+    def forward(self, A):
+        C = torch.empty(A.shape[:-1] + (self.s.shape[1],), dtype=A.dtype, device=A.device)
+        mul(A.reshape((-1, A.shape[-1])), self.B, C.view((-1, C.shape[-1])), self.s,
+            self.workspace, cute_version=self.cute_version)
+        return C
+
+    def pack(self, linear, scales):
+        """Fill B and s from a fake-quantised `torch.nn.Linear` (half weights) and its
+        scales of shape (outfeatures, groups)."""
+        if linear.weight.dtype != torch.half:
+            raise ValueError('Only `torch.half` weights are supported.')
+        s = scales.t()                 # (groups, n)
+        w = linear.weight.data.t()     # (k, n)
+        groupwise = self.groupsize != self.k
+        s_full = s.repeat_interleave(self.groupsize, dim=0) if groupwise else s
+        q = torch.clamp(torch.round(w / s_full).int() + 8, 0, 15)
+        self.B[:, :] = pack_weights(q).to(self.B.device)
+        self.s[:, :] = pack_scales(s, groupwise).to(self.s.device)
+
+
+def replace_linear(module, name_filter=lambda n: True, groupsize=-1, name=''):
+    """Recursively swap every `torch.nn.Linear` selected by `name_filter` for an
+    empty `Layer` (reference marlin.py:134-151)."""
+    if isinstance(module, Layer):
+        return
+    for child_name, child in list(module.named_children()):
+        full = f"{name}.{child_name}" if name else child_name
+        if isinstance(child, nn.Linear) and name_filter(full):
+            setattr(module, child_name,
+                    Layer(child.in_features, child.out_features, groupsize=groupsize))
+        else:
+            replace_linear(child, name_filter, groupsize=groupsize, name=full)
+
+
+def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
+    """Return code marlin_gemm would give for these sizes (no GPU touched)."""
+    return _lib.marlin_amd_check(m, n, k, groupsize, thread_k, thread_n)
+
+
+def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
+    """Kernel, grid and stream-K partition marlin_gemm would use."""
+    out = (ctypes.c_int * 6)()
+    rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
+    keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches")
+    return rc, dict(zip(keys, out))

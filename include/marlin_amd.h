@@ -1,0 +1,100 @@
+/*
+ * C ABI of the MI355X (gfx950) W4A16 Marlin GEMM library, libmarlin_amd.so.
+ *
+ * Plain pointers and sizes only.  Every buffer is a caller-owned DEVICE
+ * pointer; calls are asynchronous on the given HIP stream and return after
+ * enqueueing.  Return codes follow the reference launcher
+ * (marlin_cute_kernel.cu:4-5): 0 = ok (also for an empty problem),
+ * 1 = problem shape not compatible with the tile, 2 = no kernel for this
+ * tile / group size, and in addition 3 = the HIP runtime reported an error
+ * (the reference never checks).
+ */
+#ifndef MARLIN_AMD_H
+#define MARLIN_AMD_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MARLIN_OK 0
+#define MARLIN_ERR_PROB_SHAPE 1 /* marlin_cute_kernel.cu:4 */
+#define MARLIN_ERR_KERN_SHAPE 2 /* marlin_cute_kernel.cu:5 */
+#define MARLIN_ERR_RUNTIME 3
+#define MARLIN_ERR_GROUPS 4    /* marlin_gemm.cpp:27-28 */
+#define MARLIN_ERR_WORKSPACE 5 /* marlin_gemm.cpp:29-31 */
+
+/*
+ * FP16 x INT4 GEMM, C = A * dequant(B).  Replaces
+ *   int marlin_cute(const void *A, const void *B, void *C, void *s,
+ *                   int prob_m, int prob_n, int prob_k, void *workspace,
+ *                   int groupsize, int dev, cudaStream_t stream,
+ *                   int thread_k, int thread_n, int sms, int max_par)
+ * (declared marlin_gemm.cpp:6-9, defined marlin_cute_kernel.cu:28-115), same
+ * argument order and meaning:
+ *   A   (prob_m, prob_k) fp16 row-major
+ *   B   (prob_k/16, 2*prob_n) int32, Marlin-packed int4 (marlin.py:92-131)
+ *   C   (prob_m, prob_n) fp16 row-major, fully overwritten
+ *   s   (prob_k/groupsize, prob_n) fp16, or (1, prob_n) when groupsize == -1,
+ *       permuted as Layer.pack leaves it
+ *   workspace  at least prob_n/128*max_par int32, all zero on entry; all zero
+ *       again when the call's kernels have finished
+ *   groupsize  128 or -1 (per output column)
+ *   stream     a hipStream_t (0 = the default stream)
+ *   thread_k, thread_n   tile hints as in the reference: -1 = automatic
+ *       ((128,128) up to 16 rows, else (64,256)).  They are validated exactly
+ *       as the reference validates them but do not select the kernel.
+ *   sms        number of workgroups of the streaming kernel, -1 = automatic
+ *   max_par    only sizes the workspace contract
+ * Not re-entrant over the same workspace or the same C concurrently.
+ */
+int marlin_gemm(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
+                int prob_k, void *workspace, int groupsize, int dev, void *stream, int thread_k,
+                int thread_n, int sms, int max_par);
+
+/* Same entry under the two names the reference binding links against
+ * (marlin_gemm.cpp:6-14); both run the same kernels here. */
+int marlin_cute(const void *A, const void *B, void *C, void *s, int prob_m, int prob_n,
+                int prob_k, void *workspace, int groupsize, int dev, void *stream, int thread_k,
+                int thread_n, int sms, int max_par);
+int marlin_official(const void *A, const void *B, void *C, void *s, int prob_m, int prob_n,
+                    int prob_k, void *workspace, int groupsize, int dev, void *stream,
+                    int thread_k, int thread_n, int sms, int max_par);
+
+/*
+ * The checks of the reference's tensor-level binding `mul`
+ * (marlin_gemm.cpp:19-56) on plain sizes: derives groupsize from the number
+ * of scale rows (1 row = per-channel), rejects k not divisible into the
+ * groups (MARLIN_ERR_GROUPS) and a workspace shorter than
+ * prob_n/128*max_par entries (MARLIN_ERR_WORKSPACE), calls marlin_gemm and,
+ * on any error, writes the reference's message text into err (if non-null).
+ */
+int marlin_mul(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
+               int prob_k, int s_rows, void *workspace, long long workspace_numel, int dev,
+               void *stream, int thread_k, int thread_n, int sms, int max_par, int cute_version,
+               char *err, int err_len);
+
+/* Argument validation of marlin_gemm alone (no GPU touched): the code
+ * marlin_gemm would return for these sizes and hints. */
+int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                     int thread_n);
+
+/*
+ * How marlin_gemm would run a problem on a device with `cus` compute units:
+ * out[0] = kernel (0 = none, 1 = streaming, 2 = prefill), out[1] = workgroups,
+ * out[2] = granules per workgroup (streaming), out[3] = column tiles,
+ * out[4] = granules per column tile, out[5] = number of launches.
+ * Returns the marlin_gemm error code for the shape.
+ */
+int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                    int thread_n, int sms, int cus, int *out);
+
+/* Text of the last HIP runtime error seen by this thread ("" if none). */
+const char *marlin_amd_last_error(void);
+
+/* Library version string. */
+const char *marlin_amd_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

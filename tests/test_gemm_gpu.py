@@ -1,0 +1,256 @@
+"""GPU parity tests: the HIP path, called through the C ABI (marlin.mul ->
+marlin_mul -> marlin_gemm), against the CPU oracle on the same seeded inputs.
+
+Acceptance: dequantised weights bit-exact (probed with one-hot activation
+rows), outputs within max|C - C_ref| <= 1e-2 * max|C_ref|.  Shapes follow the
+reference's own tests (marlin_test.py:78-167) and the benchmark configs.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import _oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
+
+TOL = 1e-2  # max-abs-error <= TOL * max|ref|, fp32 accumulation
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    import marlin
+    assert torch.cuda.is_available()
+    return torch, marlin
+
+
+def gpu_gemm(env, A, B, sp, N, thread_k=-1, thread_n=-1, sms=-1, max_par=16, C_fill=None):
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    M = A.shape[0]
+    print(f"  gemm M={M} N={N} K={A.shape[1]} groups={sp.shape[0]} hints=({thread_k},{thread_n},{sms})",
+          flush=True)
+    dA = torch.from_numpy(A).to(dev)
+    dB = torch.from_numpy(B).to(dev)
+    ds = torch.from_numpy(sp).to(dev)
+    dC = torch.zeros((M, N), dtype=torch.half, device=dev)
+    if C_fill is not None:
+        dC.fill_(C_fill)
+    ws = torch.zeros(N // 128 * max_par, dtype=torch.int, device=dev)
+    marlin.mul(dA, dB, dC, ds, ws, thread_k, thread_n, sms, max_par)
+    torch.cuda.synchronize()
+    assert not ws.any().item(), "workspace must be handed back zeroed"
+    return dC.cpu().numpy()
+
+
+def check(env, M, N, K, groupsize, seed=0, **kw):
+    A, q, s, B, sp = O.make_problem(M, N, K, groupsize, seed)
+    C = gpu_gemm(env, A, B, sp, N, **kw)
+    Cref = O.gemm(A, B, sp, N, groupsize)
+    r = O.compare(C, Cref)
+    assert np.isfinite(r.max_abs_err)
+    assert r.max_abs_err <= TOL * r.max_abs_ref, (r.max_abs_err, r.max_abs_ref)
+    assert r.cosine >= 0.999
+    return r
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_dequantized_weights_bit_exact(env, groupsize):
+    """One-hot activation rows return rows of the dequantised weight matrix;
+    single-term sums leave no room for rounding differences."""
+    N, K = 256, 512
+    _, q, s, B, sp = O.make_problem(1, N, K, groupsize, seed=3)
+    W = O.dequant(B, sp, K, N, groupsize)
+    if groupsize == -1:
+        W = W * O.unpack_scales(sp, False)  # fp16(q-8) * s, one rounding
+    for rows in ([0], [5, 17, 130, 511], list(range(0, 512, 33))[:16],
+                 list(range(1, 512, 9))[:48]):
+        A = np.zeros((len(rows), K), np.float16)
+        for i, r in enumerate(rows):
+            A[i, r] = 1.0
+        C = gpu_gemm(env, A, B, sp, N)
+        assert np.array_equal(C.view(np.uint16), W[rows].view(np.uint16))
+
+
+def test_all_k_rows_bit_exact_through_identity(env):
+    """A = 64 shifted one-hot batches covers every k of a 512-deep weight."""
+    N, K = 256, 512
+    _, q, s, B, sp = O.make_problem(1, N, K, 128, seed=4)
+    W = O.dequant(B, sp, K, N, 128)
+    for base in range(0, K, 64):
+        A = np.zeros((64, K), np.float16)
+        A[np.arange(64), base + np.arange(64)] = 1.0
+        C = gpu_gemm(env, A, B, sp, N)
+        assert np.array_equal(C.view(np.uint16), W[base:base + 64].view(np.uint16))
+
+
+def test_config1_reference_case(env):
+    # BASELINE config 1 == first case of marlin_test.py:123-131
+    check(env, 16, 256, 512, 128, thread_k=128, thread_n=128)
+
+
+def test_closed_forms(env):
+    M, N, K = 16, 256, 512
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((M, K)).astype(np.float16)
+    s = rng.uniform(0.001, 0.02, (K // 128, N)).astype(np.float16)
+    q = np.full((K, N), 8, np.uint8)
+    C = gpu_gemm(env, A, O.pack_weights(q), O.pack_scales(s, True), N, C_fill=7.0)
+    assert not C.view(np.uint16).any()  # zero point everywhere -> exact zero
+    Ai = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    q = rng.integers(0, 16, (K, N), dtype=np.uint8)
+    ones = np.ones((K // 128, N), np.float16)
+    C = gpu_gemm(env, Ai, O.pack_weights(q), O.pack_scales(ones, True), N)
+    want = Ai.astype(np.int64) @ (q.astype(np.int64) - 8)
+    assert np.abs(want).max() < 2048
+    assert np.array_equal(C.astype(np.int64), want)  # exact integers
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 12, 16, 24, 32, 48, 64, 118, 128, 152])
+def test_tiles(env, m):
+    # marlin_test.py:78-84
+    for thread_k, thread_n in [(64, 256), (128, 128)]:
+        if m > 16 and thread_k == 128:
+            continue
+        check(env, m, 512, 1024, -1, seed=m, thread_k=thread_k, thread_n=thread_n)
+
+
+@pytest.mark.parametrize("k", [768, 832, 896, 64, 128, 192])
+def test_k_divisibility_and_few_stages(env, k):
+    # marlin_test.py:86-94
+    check(env, 16, 512, k, -1, seed=k, thread_k=64, thread_n=256)
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+@pytest.mark.parametrize("n,k", [(256, 512), (256, 1024), (256 * 128, 1024)])
+def test_groups(env, groupsize, n, k):
+    # marlin_test.py:123-131
+    check(env, 16, n, k, groupsize, seed=n + k, thread_k=128, thread_n=128)
+
+
+@pytest.mark.parametrize("sms", [1, 3, 7, 31, 100, 255, 256, 333, 512, 1024])
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_partition_sweep(env, sms, groupsize):
+    """Odd workgroup counts put tile boundaries in the middle of workgroups and
+    make many workgroups share a tile: exercises the fixup."""
+    check(env, 16, 1280, 1152, groupsize, seed=sms, sms=sms)
+    check(env, 48, 768, 2048, groupsize, seed=sms + 1, sms=sms)
+
+
+def test_deterministic(env):
+    A, q, s, B, sp = O.make_problem(16, 4096, 4096, 128, seed=9)
+    c1 = gpu_gemm(env, A, B, sp, 4096)
+    c2 = gpu_gemm(env, A, B, sp, 4096)
+    assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
+
+
+def test_config2_decode(env):
+    check(env, 1, 4096, 4096, 128, seed=2)
+
+
+def test_config3_mlp_pair(env):
+    check(env, 16, 11008, 4096, 128, seed=31)
+    check(env, 16, 4096, 11008, 128, seed=32)
+
+
+@pytest.mark.parametrize("m", [1, 16])
+@pytest.mark.parametrize("k,n", [(4096, 3 * 4096), (4096, 4096), (4096, 2 * 10752), (10752, 4096)])
+def test_llama7b_shapes(env, m, k, n):
+    # marlin_test.py:133-167 (7B rows; per-channel as in the reference test)
+    check(env, m, n, k, -1, seed=k + n + m, thread_k=128, thread_n=128)
+
+
+def test_config4_prefill_rows_sample(env):
+    """M=2048, N=K=4096: the oracle checks a sample of rows (the full product
+    is 69 GFLOP on the CPU); the GPU computes all of them."""
+    M, N, K = 2048, 4096, 4096
+    A, q, s, B, sp = O.make_problem(M, N, K, 128, seed=4)
+    C = gpu_gemm(env, A, B, sp, N)
+    rows = np.r_[0:8, 63:66, 127:130, 1000:1008, 2040:2048]
+    Cref = O.gemm(A[rows], B, sp, N, 128)
+    r = O.compare(C[rows], Cref)
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+    # linearity across the whole output: rows are independent, so a second
+    # call on a row permutation must give the permuted result bit for bit
+    perm = np.random.default_rng(0).permutation(M)
+    C2 = gpu_gemm(env, A[perm], B, sp, N)
+    assert np.array_equal(C2.view(np.uint16), C[perm].view(np.uint16))
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_config5_large_uneven(env, groupsize):
+    """M=64, N=28672, K=8192.  Oracle on a column slice (columns are
+    independent; a slice of the packed buffers on 128-column boundaries is a
+    valid problem of its own), GPU on the full shape."""
+    M, N, K = 64, 28672, 8192
+    A, q, s, B, sp = O.make_problem(M, N, K, groupsize, seed=5)
+    C = gpu_gemm(env, A, B, sp, N)
+    for c0 in (0, 128 * 111, N - 256):
+        Bs = np.ascontiguousarray(B[:, 2 * c0:2 * (c0 + 256)])
+        ss = np.ascontiguousarray(sp[:, c0:c0 + 256])
+        Cref = O.gemm(A, Bs, ss, 256, groupsize)
+        r = O.compare(C[:, c0:c0 + 256], Cref)
+        assert r.max_abs_err <= TOL * r.max_abs_ref, (c0, r.max_abs_err, r.max_abs_ref)
+    # zero-point weights in half of the k range must not change anything when
+    # the matching activations are garbage-free zeros: C(A) == C(A with k<4096
+    # zeroed) + C(A with k>=4096 zeroed) up to fp16 rounding of the two halves
+    A1 = A.copy(); A1[:, K // 2:] = 0
+    A2 = A.copy(); A2[:, :K // 2] = 0
+    Cs = gpu_gemm(env, A1, B, sp, N).astype(np.float32) + gpu_gemm(env, A2, B, sp, N).astype(np.float32)
+    assert np.abs(Cs - C.astype(np.float32)).max() <= TOL * np.abs(C.astype(np.float32)).max()
+
+
+def test_binding_errors_raise(env):
+    # marlin_test.py:96-121
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    m, n, k = 16, 256, 64
+    A = torch.zeros((m, k), dtype=torch.half, device=dev)
+    B = torch.zeros((k // 16, 2 * n), dtype=torch.int, device=dev)
+    s = torch.ones((1, n), dtype=torch.half, device=dev)
+    C = torch.zeros((m, n), dtype=torch.half, device=dev)
+    small_ws = torch.zeros(n // 128, dtype=torch.int, device=dev)
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int, device=dev)
+    with pytest.raises(RuntimeError, match="workspace"):
+        marlin.mul(A, B, C, s, small_ws, 128, 128, -1)
+    with pytest.raises(RuntimeError, match="not compatible with thread_k=128"):
+        marlin.mul(A, B, C, s, ws, 128, 128, -1)
+    with pytest.raises(RuntimeError, match="not compatible with thread_k=256"):
+        marlin.mul(A, B, C, s, ws, 256, 256, -1)
+    s2 = torch.zeros((2, n), dtype=torch.half, device=dev)
+    with pytest.raises(RuntimeError):
+        marlin.mul(A, B, C, s2, ws, 256, 256, -1)
+    with pytest.raises(RuntimeError, match="No kernel"):
+        marlin.mul(A, B, C, s2, ws, 64, 256, -1)  # groupsize 32
+    s3 = torch.zeros((3, n), dtype=torch.half, device=dev)
+    with pytest.raises(RuntimeError, match="groups"):
+        marlin.mul(A, B, C, s3, ws, 64, 256, -1)
+
+
+def test_layer_forward_matches_oracle(env):
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    k, n, m = 512, 256, 8
+    rng = np.random.default_rng(21)
+    w = rng.standard_normal((k, n)).astype(np.float16)
+    for groupsize in (128, -1):
+        q, s, ref = O.gen_quant4(w, groupsize)
+        linear = torch.nn.Linear(k, n, bias=False)
+        linear.weight.data = torch.from_numpy(ref).t().contiguous()
+        layer = marlin.Layer(k, n, groupsize=groupsize)
+        layer.pack(linear, torch.from_numpy(s).t().contiguous())
+        assert np.array_equal(layer.B.numpy(), O.pack_weights(q))
+        layer = layer.to(dev)
+        A = rng.standard_normal((2, m // 2, k)).astype(np.float16)
+        out = layer(torch.from_numpy(A).to(dev))
+        torch.cuda.synchronize()
+        assert out.shape == (2, m // 2, n)
+        Cref = O.gemm(A.reshape(m, k), O.pack_weights(q), O.pack_scales(s, groupsize != -1), n,
+                      groupsize)
+        r = O.compare(out.cpu().numpy().reshape(m, n), Cref)
+        assert r.max_abs_err <= TOL * r.max_abs_ref
