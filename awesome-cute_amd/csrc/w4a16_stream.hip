@@ -1,7 +1,7 @@
 // Streaming W4A16 kernel for at most 64 activation rows (decode and small
-// batch): the weight stream is the roofline, so every wave keeps a deep queue
-// of 128-bit weight loads in flight straight into registers and never waits
-// on another wave inside the main loop.
+// batch): the weight stream is the roofline, so every wave keeps a ring of
+// 128-bit weight loads in flight straight into registers and never waits on
+// another wave inside the main loop.
 //
 // Work split (see make_stream_plan): a launch is NT*KG granules of
 // 128 columns x 64 k.  A workgroup (4 waves) owns a contiguous run of
@@ -11,9 +11,53 @@
 // the partial sums meet in global memory: everybody stores fp32 partials,
 // bumps the tile's counter, and the last arrival adds all partials in
 // workgroup order and writes C.  Nobody ever spins.
+//
+// All global reads are buffer loads issued unconditionally, DEPTH granules
+// ahead, so that the hardware's in-order load counter can be waited on
+// exactly; a granule that does not exist is requested at an out-of-range
+// offset, which returns zeros without touching memory.  The ring keeps
+// running across column tiles: the first granules of the next tile are in
+// flight while the current tile is reduced and written.
 #include "w4a16_common.hpp"
 
+// Optional phase timestamps for tuning builds; empty in the library build.
+#ifndef W4A16_STAMP_DECL
+#define W4A16_STAMP_DECL
+#define W4A16_STAMP(i)
+#endif
+
 namespace w4a16 {
+
+namespace {
+
+constexpr int kOob = (int)0x80000000;  // offset past any buffer (sizes are < 2 GiB)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+
+// s_waitcnt vmcnt(0) with the other counters left alone (gfx9 encoding)
+constexpr int kWaitVm0 = 0x0F70;
+
+typedef unsigned long long u64;
+
+// 16 bytes as two 64-bit device-scope accesses: stores are written through to
+// memory shared by all XCDs, loads never return a line cached by this XCD's L2.
+__device__ __forceinline__ void store_device_scope(f4* p, f4 v) {
+  u64 lo = ((u64)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]);
+  u64 hi = ((u64)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
+  __hip_atomic_store((u64*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((u64*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f4 load_device_scope(const f4* p) {
+  u64 lo = __hip_atomic_load((const u64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  u64 hi = __hip_atomic_load((const u64*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  f4 r = {__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
+          __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
+  return r;
+}
+
+}  // namespace
 
 template <int MB, bool GROUP, int DEPTH>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
@@ -22,8 +66,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) char smem[32768];
   __shared__ int s_ticket;
 
+  W4A16_STAMP_DECL
   const int tid = threadIdx.x;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int lane = tid & 63;
   const int kg = lane >> 4;  // k group of the MFMA operand layout
   const int nu = lane & 15;  // column slot (weights) / row (activations)
@@ -33,26 +78,30 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   plan.KG = p.K / kGranuleK;
   plan.gpb = p.gpb;
   plan.grid = (int)gridDim.x;
-  const int total = plan.NT * plan.KG;
+  const int KG = plan.KG;
+  const int total = plan.NT * KG;
   const int u0 = (int)blockIdx.x * plan.gpb;
   if (u0 >= total) return;
   const int u1 = min(total, u0 + plan.gpb);
 
-  const i4* __restrict__ B4 = (const i4*)p.B;
-  const i4* __restrict__ A4 = (const i4*)p.A;
-  const i4* __restrict__ S4 = (const i4*)p.S;
-  const size_t b_row = (size_t)(p.N / 2);  // int4 per row of B
-  const size_t a_row = (size_t)(p.K / 8);  // int4 per row of A
+  const __amdgpu_buffer_rsrc_t rB = make_rsrc(p.B, (unsigned)p.K * (unsigned)(p.N / 2));
+  const __amdgpu_buffer_rsrc_t rA = make_rsrc(p.A, (unsigned)p.M * (unsigned)p.K * 2u);
+  const __amdgpu_buffer_rsrc_t rS =
+      make_rsrc(p.S, (unsigned)(GROUP ? p.K / 128 : 1) * (unsigned)p.N * 2u);
+  const int b_row = p.N * 8;  // bytes per row of B (16 k-values of every column)
 
-  // activation staging: lane (row = lane/4, ax = lane%4) fetches chunks ax and
-  // ax+4 (16 bytes each) of the 128-byte k run of its row
+  // per-lane parts of the addresses; the rest is wave-uniform
+  const int b_lane = 64 * nu + 16 * kg;
+  const int s_lane = 16 * nu;
+  // activation staging: lane (row = lane/4, ax = lane%4) fetches 16-byte
+  // chunks ax and ax+4 of the 128-byte k run of its row
   const int ax = lane & 3;
-  size_t a_off[MB];
+  int a_lane[MB];
 #pragma unroll
   for (int i = 0; i < MB; i++) {
     int r = 16 * i + (lane >> 2);
     r = r < p.M ? r : p.M - 1;  // rows past M are never written back
-    a_off[i] = (size_t)r * a_row + ax;
+    a_lane[i] = r * p.K * 2 + 16 * ax;
   }
   char* lds_a = smem + wave * (MB * 2048);
   // write position of dword kg' of a chunk: [step][kg'][row][ax]
@@ -62,88 +111,86 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 
   const DequantConsts dc;
 
-  for (int t = u0 / plan.KG; t * plan.KG < u1; ++t) {
-    const int seg_a = max(u0, t * plan.KG) - t * plan.KG;
-    const int seg_e = min(u1, (t + 1) * plan.KG) - t * plan.KG;
-    const int n_my = (seg_e - seg_a > wave) ? ((seg_e - seg_a - wave + 3) >> 2) : 0;
-    const int kq0 = seg_a + wave;  // my granules: kq0, kq0+4, ...
+  i4 bq[DEPTH][4];
+  i4 sq[DEPTH];
+  i4 aq[DEPTH][MB][2];
 
-    const i4* bptr = B4 + (size_t)64 * t + 4 * nu + kg;
-    const i4* sptr = S4 + (size_t)16 * t + nu;
+  // request granule kq of tile t into ring slot `slot`; straight-line code, so
+  // that every turn of the ring issues exactly the same loads in the same order
+  auto issue = [&](int slot, int t, int kq, bool valid) {
+    __builtin_amdgcn_sched_barrier(0);
+    const int inv = valid ? 0 : kOob;
+    const int vb = b_lane | inv;
+    const int sb = (4 * kq) * b_row + 1024 * t;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      bq[slot][r] = __builtin_amdgcn_raw_buffer_load_b128(rB, vb, sb + r * b_row, 2);
+    if (GROUP)
+      sq[slot] = __builtin_amdgcn_raw_buffer_load_b128(rS, s_lane | inv,
+                                                       ((kq >> 1) * p.N + kTileN * t) * 2, 0);
+#pragma unroll
+    for (int i = 0; i < MB; i++) {
+      aq[slot][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq, 0);
+      aq[slot][i][1] =
+          __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq + 64, 0);
+    }
+    // keep the groups in issue order: the in-order load counter is only exact
+    // if a slot's loads are never moved behind those of a later slot
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-    f4 acc[MB][8];
+  f4 acc[MB][8];
+  auto clear_acc = [&]() {
 #pragma unroll
     for (int i = 0; i < MB; i++)
 #pragma unroll
       for (int j = 0; j < 8; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+  };
 
-    i4 bq[DEPTH][4];
-    i4 sq[DEPTH];
-    i4 aq[DEPTH][MB][2];
-
-    auto issue = [&](int slot, int kq) {
+  auto compute = [&](int slot) {
+    // activations: registers -> LDS in MFMA k-slot order
 #pragma unroll
-      for (int r = 0; r < 4; r++)
-        bq[slot][r] = __builtin_nontemporal_load(bptr + (size_t)(4 * kq + r) * b_row);
-      if (GROUP) sq[slot] = sptr[(size_t)(kq >> 1) * (p.N / 8)];
+    for (int i = 0; i < MB; i++)
 #pragma unroll
-      for (int i = 0; i < MB; i++) {
-        aq[slot][i][0] = A4[a_off[i] + 8 * kq];
-        aq[slot][i][1] = A4[a_off[i] + 8 * kq + 4];
-      }
-    };
-
-    auto compute = [&](int slot) {
-      // activations: registers -> LDS in MFMA k-slot order
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+          *(int*)(lds_a + i * 2048 + h * 1024 + g * 256 + a_wr) = aq[slot][i][h][g];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      h8 af[MB];
 #pragma unroll
       for (int i = 0; i < MB; i++)
+        af[i] = __builtin_bit_cast(h8, *(const i4*)(lds_a + i * 2048 + h * 1024 + a_rd));
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+      for (int j = 0; j < 4; j++) {
+        h2 s2 = GROUP ? as_h2(sq[slot][j]) : (h2){(half_t)1.f, (half_t)1.f};
+        h2 l0, h0, l1, h1, m0, n0, m1, n1;
+        dequant_word<GROUP>(bq[slot][2 * h][j], s2, dc, l0, h0, l1, h1);
+        dequant_word<GROUP>(bq[slot][2 * h + 1][j], s2, dc, m0, n0, m1, n1);
+        h8 w0 = make_h8(l0, h0, m0, n0);
+        h8 w1 = make_h8(l1, h1, m1, n1);
 #pragma unroll
-          for (int g = 0; g < 4; g++)
-            *(int*)(lds_a + i * 2048 + h * 1024 + g * 256 + a_wr) = aq[slot][i][h][g];
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        h8 af[MB];
-#pragma unroll
-        for (int i = 0; i < MB; i++)
-          af[i] = __builtin_bit_cast(h8, *(const i4*)(lds_a + i * 2048 + h * 1024 + a_rd));
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          h2 s2 = GROUP ? as_h2(sq[slot][j]) : (h2){(half_t)1.f, (half_t)1.f};
-          h2 l0, h0, l1, h1, m0, n0, m1, n1;
-          dequant_word<GROUP>(bq[slot][2 * h][j], s2, dc, l0, h0, l1, h1);
-          dequant_word<GROUP>(bq[slot][2 * h + 1][j], s2, dc, m0, n0, m1, n1);
-          h8 w0 = make_h8(l0, h0, m0, n0);
-          h8 w1 = make_h8(l1, h1, m1, n1);
-#pragma unroll
-          for (int i = 0; i < MB; i++) {
-            acc[i][2 * j] =
-                __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, af[i], acc[i][2 * j], 0, 0, 0);
-            acc[i][2 * j + 1] =
-                __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, af[i], acc[i][2 * j + 1], 0, 0, 0);
-          }
-        }
-      }
-    };
-
-#pragma unroll
-    for (int d = 0; d < DEPTH; d++)
-      if (d < n_my) issue(d, kq0 + 4 * d);
-    for (int base = 0; base < n_my; base += DEPTH) {
-#pragma unroll
-      for (int d = 0; d < DEPTH; d++) {
-        if (base + d < n_my) {
-          compute(d);
-          if (base + d + DEPTH < n_my) issue(d, kq0 + 4 * (base + d + DEPTH));
+        for (int i = 0; i < MB; i++) {
+          acc[i][2 * j] =
+              __builtin_amdgcn_mfma_f32_16x16x32_f16(w0, af[i], acc[i][2 * j], 0, 0, 0);
+          acc[i][2 * j + 1] =
+              __builtin_amdgcn_mfma_f32_16x16x32_f16(w1, af[i], acc[i][2 * j + 1], 0, 0, 0);
         }
       }
     }
+  };
 
+  // Finish column tile t: sum the four waves, meet the other workgroups that
+  // share the tile, write C.  Every wave calls this exactly once per tile of
+  // the workgroup, in tile order.
+  auto finish = [&](int t) {
     // ---- sum the four waves; wave w ends up owning the 16-column groups
     // (j = w, h = 0/1) of every row block
     f4 res[MB][2];
+    W4A16_STAMP(3)
     __syncthreads();
+    W4A16_STAMP(4)
 #pragma unroll
     for (int i = 0; i < MB; i++) {
       f4* red = (f4*)smem;
@@ -160,7 +207,13 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       __syncthreads();
     }
 
-    // ---- meet the other workgroups of this tile, if any
+    W4A16_STAMP(5)
+    // ---- meet the other workgroups of this tile, if any.  Partial sums
+    // travel through device-scope (write-through / always-refetched) stores
+    // and loads, so no cache write-back or invalidation is needed: a wave
+    // waits until its own stores are acknowledged, the barrier collects the
+    // four waves, and only then does thread 0 take the tile's ticket.  Whoever
+    // draws the last ticket knows every other partial has already landed.
     const int bf = tile_first_block(plan, t);
     const int bl = tile_last_block(plan, t);
     bool writer = true;
@@ -171,44 +224,58 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       for (int i = 0; i < MB; i++)
         if (16 * i + nu < p.M) {
 #pragma unroll
-          for (int h = 0; h < 2; h++) mine[((i * 4 + wave) * 2 + h) * 64 + lane] = res[i][h];
+          for (int h = 0; h < 2; h++)
+            store_device_scope(&mine[((i * 4 + wave) * 2 + h) * 64 + lane], res[i][h]);
         }
-      __threadfence();  // partials visible device-wide before the ticket
+      __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
       __syncthreads();
       if (tid == 0)
         s_ticket = __hip_atomic_fetch_add(&p.locks[t], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
+      W4A16_STAMP(6)
       writer = (s_ticket == bl - bf);
       if (writer) {
-        __threadfence();  // see everybody else's partials
+        // add the partials in workgroup order (deterministic), fetching them
+        // eight workgroups at a time so that the loads overlap
 #pragma unroll
         for (int i = 0; i < MB; i++) {
           if (16 * i + nu < p.M) {
-            f4 sum[2];
-            for (int b = bf; b <= bl; b++) {
-              f4 v[2];
-              if (b == (int)blockIdx.x) {
-                v[0] = res[i][0];
-                v[1] = res[i][1];
-              } else {
-                const f4* theirs =
-                    (const f4*)p.scratch + (size_t)partial_slot(plan, b, t) * slot_f4;
-                v[0] = theirs[((i * 4 + wave) * 2 + 0) * 64 + lane];
-                v[1] = theirs[((i * 4 + wave) * 2 + 1) * 64 + lane];
+            f4 sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            for (int b0 = bf; b0 <= bl; b0 += 8) {
+              f4 v[8][2];
+#pragma unroll
+              for (int u = 0; u < 8; u++) {
+                const int b = b0 + u;
+                if (b <= bl && b != (int)blockIdx.x) {
+                  const f4* theirs =
+                      (const f4*)p.scratch + (size_t)partial_slot(plan, b, t) * slot_f4;
+                  v[u][0] = load_device_scope(&theirs[((i * 4 + wave) * 2 + 0) * 64 + lane]);
+                  v[u][1] = load_device_scope(&theirs[((i * 4 + wave) * 2 + 1) * 64 + lane]);
+                } else {
+                  v[u][0] = res[i][0];
+                  v[u][1] = res[i][1];
+                }
               }
-              sum[0] = (b == bf) ? v[0] : sum[0] + v[0];
-              sum[1] = (b == bf) ? v[1] : sum[1] + v[1];
+#pragma unroll
+              for (int u = 0; u < 8; u++) {
+                if (b0 + u <= bl) {
+                  sum[0] = (b0 + u == bf) ? v[u][0] : sum[0] + v[u][0];
+                  sum[1] = (b0 + u == bf) ? v[u][1] : sum[1] + v[u][1];
+                }
+              }
             }
             res[i][0] = sum[0];
             res[i][1] = sum[1];
           }
         }
-        if (tid == 0) p.locks[t] = 0;  // counters are handed back zeroed
+        if (tid == 0)  // counters are handed back zeroed
+          __hip_atomic_store(&p.locks[t], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();  // s_ticket is reused by the next tile
     }
 
+    W4A16_STAMP(7)
     // ---- write C (fp16); per-channel mode scales the rounded result
     if (writer) {
       half_t* C = (half_t*)p.C;
@@ -234,13 +301,79 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         }
       }
     }
+  };
+
+  // My granules are u0 + wave, u0 + wave + 4, ... < u1, walked in one flat
+  // sequence across column tiles; (t, kq) are kept incrementally for the
+  // compute position and for the issue position DEPTH granules ahead.
+  const int n_mine = (u1 - u0 > wave) ? ((u1 - u0 - wave + 3) >> 2) : 0;
+  const int t_first = u0 / KG;
+  const int t_last = (u1 - 1) / KG;
+  int it = t_first, ikq = u0 - t_first * KG + wave;  // issue position
+  while (ikq >= KG) {
+    ikq -= KG;
+    ++it;
   }
+  int ct = it, ckq = ikq;  // compute position
+  int cur_tile = t_first;  // tile whose sums are in acc
+  clear_acc();
+
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) {
+    issue(d, it, ikq, d < n_mine);
+    ikq += 4;
+    while (ikq >= KG) {
+      ikq -= KG;
+      ++it;
+    }
+  }
+
+  W4A16_STAMP(1)
+  for (int base = 0; base < n_mine; base += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      const int i = base + d;
+      if (i < n_mine) {
+        // entering a new tile: hand over the tiles behind me first
+        while (cur_tile < ct) {
+          finish(cur_tile);
+          ++cur_tile;
+          clear_acc();
+        }
+      }
+      compute(d);  // a granule past the end is all zeros and adds nothing
+      if (i == 0) { W4A16_STAMP(2) }
+      ckq += 4;
+      while (ckq >= KG) {
+        ckq -= KG;
+        ++ct;
+      }
+      issue(d, it, ikq, i + DEPTH < n_mine);
+      ikq += 4;
+      while (ikq >= KG) {
+        ikq -= KG;
+        ++it;
+      }
+    }
+  }
+  while (cur_tile <= t_last) {
+    finish(cur_tile);
+    ++cur_tile;
+    clear_acc();
+  }
+  W4A16_STAMP(8)
 }
 
 template <int MB, bool GROUP>
 static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
-  constexpr int DEPTH = MB <= 2 ? 4 : 3;
-  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), 0, stream, a);
+  // ring depth: shallow when a wave only ever sees a couple of granules
+  const int per_wave = (a.gpb + 3) / 4;
+  if (per_wave <= 2) {
+    hipLaunchKernelGGL((stream_kernel<MB, GROUP, 2>), dim3(grid), dim3(256), 0, stream, a);
+  } else {
+    constexpr int DEPTH = MB <= 2 ? 4 : 3;
+    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), 0, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

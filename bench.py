@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A16 Marlin GEMM hot path on one MI355X.
+
+A step is one GEMM call (marlin.mul -> C ABI -> HIP kernel) on synthetic,
+seeded inputs already resident in HBM.  Memory-bound shapes rotate over enough
+distinct weight/scale buffers to exceed the 256 MB Infinity Cache, so the
+figure is an HBM figure and not a cache figure.  The K timed steps are captured
+in one HIP graph (kernel launches only) and bracketed by HIP events on the
+launch stream, so the host's launch cost is not part of the kernel's number;
+the eager (one host call per step) rate is reported next to it.
+
+Prints ONE JSON line: the headline workload is BASELINE config 2 (decode,
+M=1, N=K=4096, group 128), with `roofline` for its kernel and `cpu_baseline`
+from the CPU oracle; `shapes` carries the other points of the metric
+(M=16 and M=2048 at N=K=4096) measured the same way.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+MALL_BYTES = 256 << 20
+
+SHAPES = {
+    # name: (M, N, K, groupsize, bound)
+    "decode": (1, 4096, 4096, 128, "hbm"),          # BASELINE configs[1]
+    "batch16": (16, 4096, 4096, 128, "hbm"),        # metric's M=16 point
+    "prefill": (2048, 4096, 4096, 128, "mfma"),     # BASELINE configs[3]
+    "mlp_up": (16, 11008, 4096, 128, "hbm"),        # configs[2]
+    "mlp_down": (16, 4096, 11008, 128, "hbm"),
+    "large_g128": (64, 28672, 8192, 128, "hbm"),    # configs[4]
+    "large_chan": (64, 28672, 8192, -1, "hbm"),
+}
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def build_inputs(torch, O, M, N, K, groupsize, nbuf, seed=0):
+    import numpy as np
+    dev = torch.device("cuda:0")
+    A, q, s, B, sp = O.make_problem(M, N, K, groupsize, seed)
+    dA = torch.from_numpy(A).to(dev)
+    dBs, dSs = [], []
+    rng = np.random.default_rng(seed + 1)
+    hB = torch.from_numpy(B)
+    hS = torch.from_numpy(sp)
+    for i in range(nbuf):
+        if i == 0:
+            dBs.append(hB.to(dev))
+            dSs.append(hS.to(dev))
+        else:
+            # distinct memory with the same value distribution: a row rotation
+            # of the packed buffers (uniform nibbles stay uniform)
+            dBs.append(torch.roll(dBs[0], shifts=i, dims=0).contiguous())
+            dSs.append(torch.roll(dSs[0], shifts=i, dims=1).contiguous())
+    dC = torch.zeros((M, N), dtype=torch.half, device=dev)
+    ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+    return (A, B, sp), dA, dBs, dSs, dC, ws
+
+
+def time_shape(torch, marlin, O, name, steps, warmup, check=True):
+    M, N, K, g, bound = SHAPES[name]
+    weight_bytes = K * N // 2
+    nbuf = max(2, -(-2 * MALL_BYTES // weight_bytes)) if bound == "hbm" else 2
+    nbuf = min(nbuf, 96)
+    host, dA, dBs, dSs, dC, ws = build_inputs(torch, O, M, N, K, g, nbuf)
+
+    def call(i):
+        marlin.mul(dA, dBs[i % nbuf], dC, dSs[i % nbuf], ws)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(max(warmup, 3)):
+            call(i)
+        side.synchronize()
+        if check:
+            import numpy as np
+            call(0)
+            side.synchronize()
+            A, B, sp = host
+            rows = slice(0, min(M, 4))
+            ref = O.gemm(A[rows], B, sp, N, g)
+            r = O.compare(dC[rows].cpu().numpy(), ref)
+            assert r.max_abs_err <= 1e-2 * r.max_abs_ref, (name, r.max_abs_err, r.max_abs_ref)
+            assert not ws.any().item()
+        # eager: one host call per step
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        side.synchronize()
+        t0 = time.perf_counter()
+        e0.record(side)
+        for i in range(steps):
+            call(i)
+        e1.record(side)
+        side.synchronize()
+        eager_ms = (time.perf_counter() - t0) * 1e3 / steps
+        eager_dev_ms = e0.elapsed_time(e1) / steps
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for i in range(steps):
+            call(i)
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    cur = torch.cuda.current_stream()
+    g0.record(cur)
+    graph.replay()
+    g1.record(cur)
+    torch.cuda.synchronize()
+    ms = g0.elapsed_time(g1) / steps
+
+    flops = 2.0 * M * N * K
+    res = {
+        "name": name, "M": M, "N": N, "K": K, "groupsize": g,
+        "ms_per_step": ms, "us_per_launch": ms * 1e3,
+        "eager_ms_per_step": eager_ms, "eager_device_ms_per_step": eager_dev_ms,
+        "weight_GBps": weight_bytes / (ms * 1e-3) / 1e9,
+        "tflops": flops / (ms * 1e-3) / 1e12,
+        "weight_buffers_rotated": nbuf,
+    }
+    if bound == "hbm":
+        ach = res["weight_GBps"]
+        res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": ach / HBM_PEAK_GBPS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+    else:
+        ach = res["tflops"]
+        res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": MFMA_FP16_PEAK_TFLOPS,
+                           "unit": "TFLOP/s", "frac": ach / MFMA_FP16_PEAK_TFLOPS,
+                           "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+    return res
+
+
+def cpu_baseline(O, name, budget_s=12.0):
+    """The CPU oracle (a port: the reference has no CPU implementation of this
+    path) on the same workload, repeated until about budget_s of CPU time."""
+    M, N, K, g, _ = SHAPES[name]
+    A, q, s, B, sp = O.make_problem(M, N, K, g, 0)
+    threads = O.lib.w4a16_ref_max_threads()
+    O.gemm(A, B, sp, N, g)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        O.gemm(A, B, sp, N, g)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or reps >= 200:
+            break
+    per = dt / reps
+    return {"value": (K * N // 2) / per / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} full GEMMs of {name} (M={M} N={N} K={K} group={g}), "
+                      f"{per * 1e3:.1f} ms each, dequantise + fp32 GEMM, OpenMP",
+            "tflops": 2.0 * M * N * K / per / 1e12}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--shape", default="headline",
+                    help="headline (decode + batch16 + prefill) or one of: " + ", ".join(SHAPES))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 "
+                 "(column-parallel sharding is described in DESIGN.md, not built)")
+
+    import torch
+    import marlin
+    import _oracle as O
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    if args.shape == "headline":
+        main_name, others = "decode", ["batch16", "prefill"]
+    else:
+        main_name, others = args.shape, []
+
+    def steps_for(name):
+        # keep the captured graph and the run time bounded for the big shapes
+        M, N, K, g, _ = SHAPES[name]
+        gflop = 2.0 * M * N * K / 1e9
+        cap = 2000 if gflop < 2 else (400 if gflop < 40 else 100)
+        return max(1, min(args.steps, cap)) if name != main_name else args.steps
+
+    head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup)
+    shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup) for n in others]
+
+    M, N, K, g, bound = SHAPES[main_name]
+    out = {
+        "metric": "w4a16_gemm_weight_hbm_GBps" if bound == "hbm" else "w4a16_gemm_tflops",
+        "value": head["weight_GBps"] if bound == "hbm" else head["tflops"],
+        "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{main_name}: M={M} N={N} K={K} groupsize={g} W4A16 GEMM",
+                   "weight_buffers_rotated": head["weight_buffers_rotated"],
+                   "timing": "K launches in one HIP graph, HIP events on the launch stream"},
+        "tflops": head["tflops"], "weight_GBps": head["weight_GBps"],
+        "eager_ms_per_step": head["eager_ms_per_step"],
+        "roofline": head["roofline"],
+        "shapes": shapes,
+        "reference_published": {"RTX4090_marlin_cute_us": 8.714, "shape": "M=1 N=4096 K=4096 g=128",
+                                "note": "cache-warm kernel time on other hardware, not comparable"}
+        if main_name == "decode" else None,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(O, main_name)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
