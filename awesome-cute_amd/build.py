@@ -5,7 +5,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmarlin_amd.so")
-SOURCES = ["marlin_host.hip", "w4a16_stream.hip"]
+SOURCES = ["marlin_host.hip", "w4a16_stream.hip", "w4a16_prefill.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

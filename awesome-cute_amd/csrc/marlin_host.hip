@@ -119,6 +119,14 @@ constexpr int kStreamMaxRows = 64;
 
 Plan make_plan(int m, int n, int k, int sms, int cus) {
   Plan pl;
+  if (m > kStreamMaxRows) {
+    // MFMA-bound: one workgroup per 128 x 256 tile of C
+    pl.kernel = 2;
+    pl.grid = ceil_div(m, 128) * (n / 256);
+    pl.sp = make_stream_plan(n, k, 1);
+    pl.launches = 1;
+    return pl;
+  }
   pl.kernel = 1;
   int want = sms > 0 ? sms : cus * env_int("MARLIN_AMD_STREAM_WG_PER_CU", 1);
   if (want > kMaxStreamGrid) want = kMaxStreamGrid;
@@ -151,8 +159,22 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0) {
     Plan pl = make_plan(m, n, k, sms, cus);
-    float* scratch = scratch_for(dev, stream);
-    if (scratch) {
+    float* scratch = pl.kernel == 1 ? scratch_for(dev, stream) : nullptr;
+    if (pl.kernel == 2) {
+      GemmArgs a;
+      a.A = A;
+      a.B = B;
+      a.C = C;
+      a.S = s;
+      a.M = m;
+      a.N = n;
+      a.K = k;
+      a.locks = (int*)workspace;
+      a.scratch = nullptr;
+      a.gpb = 0;
+      rc = launch_prefill(a, groupsize != -1, stream);
+      if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
+    } else if (scratch) {
       rc = MARLIN_OK;
       for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
         GemmArgs a;
