@@ -1,22 +1,33 @@
 // Prefill W4A16 kernel (more than 64 activation rows): MFMA-bound, so the
 // design minimises everything that competes with the matrix pipe.
 //
-// One workgroup (4 waves, one per SIMD) owns a 128-row x 256-column tile of C
-// over the whole k range.  Wave w keeps a 128 x 64 fp32 accumulator (128
-// registers): columns 16j+8h+c of the two 64-column blocks 2p, 2p+1 with
-// p = w/2 and j in {2(w%2), 2(w%2)+1}.
+// One workgroup of 8 waves (two per SIMD) owns a 128-row x 256-column tile of
+// C.  Waves 0-3 run the first half of the k range and waves 4-7 the second
+// half over the same tile, and the two halves are added through LDS at the
+// end.  Two waves per SIMD matter: a wave cannot issue its own unpack/LDS
+// instructions under its own MFMAs, but the other wave's run there for free.
+// Within a half, wave w keeps a 128 x 64 fp32 accumulator (128 registers):
+// columns 16j+8h+c of the two 64-column blocks 2p, 2p+1 with p = w/2 and
+// j in {2(w%2), 2(w%2)+1}.
 //   - Weights never touch LDS: each lane reads the 8 bytes of its Marlin
 //     16-byte piece that belong to its two 16-column groups straight from
 //     global memory (L2-resident after the first row tile), unpacks them in
 //     registers and feeds them to the MFMA as the first operand.  One unpack
 //     serves eight MFMAs (the eight 16-row blocks).
-//   - Activations are shared by the four waves: the workgroup stages a
-//     128 x 64 fp16 slab per k stage through LDS, double buffered, stored in
-//     the k-slot order the weight layout dictates so that an operand is one
-//     conflict-free ds_read_b128.
+//   - Activations are shared by the four waves of a half: they stage a
+//     128 x 64 fp16 slab per k stage through a ring of three LDS buffers,
+//     stored in the k-slot order the weight layout dictates so that an
+//     operand is one conflict-free ds_read_b128.
 // Per 32-deep k step a wave issues 32 MFMAs, 8 LDS reads and the unpack of 4
-// weight words (about 52 VALU instructions).
+// weight words (about 52 VALU instructions), software-pipelined one step
+// ahead.
 #include "w4a16_common.hpp"
+
+// Tuning builds may remap the k stage that is fetched (e.g. to a cache-hot
+// one); the library build fetches the stage it computes.
+#ifndef W4A16_PF_K
+#define W4A16_PF_K(s) (s)
+#endif
 
 namespace w4a16 {
 
@@ -25,8 +36,10 @@ namespace {
 constexpr int kPfTileM = 128;
 constexpr int kPfTileN = 256;
 constexpr int kPfStageK = 64;
-constexpr int kPfStepBytes = 4 * 128 * 16 + 128;       // one 32-deep k step of the slab (+pad)
-constexpr int kPfStageBytes = 2 * kPfStepBytes;        // two steps per stage
+constexpr int kPfStepBytes = 4 * 128 * 16 + 128;  // one 32-deep k step of the slab (+pad)
+constexpr int kPfStageBytes = 2 * kPfStepBytes;   // two steps per stage
+constexpr int kPfRing = 3;                        // slabs in LDS per k half
+constexpr int kPfLdsBytes = 2 * kPfRing * kPfStageBytes;
 constexpr int kOobPf = (int)0x80000000;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigned bytes) {
@@ -36,10 +49,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigne
 }  // namespace
 
 template <bool GROUP>
-__global__ __launch_bounds__(256) void prefill_kernel(GemmArgs p, int tiles_m, int tiles_n) {
-  __shared__ __attribute__((aligned(16))) char smem[2 * kPfStageBytes];
+__global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) char smem_all[];  // kPfLdsBytes
 
-  const int tid = threadIdx.x;
+  const int kh = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);  // k half
+  const int tid = threadIdx.x & 255;  // thread within the half
+  char* smem = smem_all + kh * (kPfRing * kPfStageBytes);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int kg = lane >> 4;
@@ -82,29 +97,47 @@ __global__ __launch_bounds__(256) void prefill_kernel(GemmArgs p, int tiles_m, i
   const int a_rd = kg * 2048 + nu * 16;
 
   const DequantConsts dc;
-  const int stages = p.K / kPfStageK;
+  // this half's stages: [s_begin, s_end) of the K/64 stages; the loop runs the
+  // same count in both halves (a stage past s_end fetches zeros)
+  const int stages_all = p.K / kPfStageK;
+  const int half_stages = (stages_all + 1) >> 1;
+  const int s_begin = kh * half_stages;
+  const int s_end = kh ? stages_all : half_stages;
+  const int stages = half_stages;
 
-  i4 areg[4];   // slab of the stage after next, in flight
-  i2 breg[2][4];  // weight words of this stage and the next: 4 rows x 8 bytes
+  i4 areg[4];     // slab of the stage after next, in flight
+  i2 breg[2][4];  // weight words of two stages: 4 rows x 8 bytes each
   i2 sreg[2];
 
   auto issue_b = [&](int slot, int s) {
-    const int inv = s < stages ? 0 : kOobPf;
+#ifdef W4A16_PF_SKIP_B
+    return;
+#endif
+    const int sg = s_begin + s;  // stage in the whole k range
+    const int inv = sg < s_end ? 0 : kOobPf;
 #pragma unroll
     for (int r = 0; r < 4; r++)
-      breg[slot][r] =
-          __builtin_amdgcn_raw_buffer_load_b64(rB, b_lane | inv, (4 * s + r) * b_row, 0);
+      breg[slot][r] = __builtin_amdgcn_raw_buffer_load_b64(rB, b_lane | inv,
+                                                           (4 * W4A16_PF_K(sg) + r) * b_row, 0);
     if (GROUP)
-      sreg[slot] = __builtin_amdgcn_raw_buffer_load_b64(rS, s_lane | inv, (s >> 1) * p.N * 2, 0);
+      sreg[slot] = __builtin_amdgcn_raw_buffer_load_b64(rS, s_lane | inv,
+                                                        (W4A16_PF_K(sg) >> 1) * p.N * 2, 0);
   };
   auto issue_a = [&](int s) {
-    const int inv = s < stages ? 0 : kOobPf;
+#ifdef W4A16_PF_SKIP_A
+    return;
+#endif
+    const int sg = s_begin + s;
+    const int inv = sg < s_end ? 0 : kOobPf;
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, s * 128, 0);
+      areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
   };
-  auto store_a = [&](int buf) {
-    char* base = smem + buf * kPfStageBytes + a_wr;
+  auto store_a = [&](int ring) {
+#ifdef W4A16_PF_SKIP_ST
+    return;
+#endif
+    char* base = smem + ring * kPfStageBytes + a_wr;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -117,47 +150,111 @@ __global__ __launch_bounds__(256) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
-  auto step = [&](int buf, int slot, int h) {
-    h8 w[4];
-#pragma unroll
-    for (int j2 = 0; j2 < 2; j2++) {
-      h2 s2 = GROUP ? as_h2(sreg[slot][j2]) : (h2){(half_t)1.f, (half_t)1.f};
-      h2 l0, h0, l1, h1, m0_, n0_, m1_, n1_;
-      dequant_word<GROUP>(breg[slot][2 * h][j2], s2, dc, l0, h0, l1, h1);
-      dequant_word<GROUP>(breg[slot][2 * h + 1][j2], s2, dc, m0_, n0_, m1_, n1_);
-      w[2 * j2] = make_h8(l0, h0, m0_, n0_);
-      w[2 * j2 + 1] = make_h8(l1, h1, m1_, n1_);
-    }
-    const char* base = smem + buf * kPfStageBytes + h * kPfStepBytes + a_rd;
+  h8 w[2][4];  // unpacked weights of the current and the next k step
+  i4 af[4];    // ring of activation operands, three ahead of the MFMAs
+#ifdef W4A16_PF_INIT
+  for (int i = 0; i < 4; i++) { areg[i] = (i4){tid, 1, 2, 3}; af[i] = (i4){tid, 5, 6, 7}; }
+  for (int i = 0; i < 2; i++) for (int r = 0; r < 4; r++) { breg[i][r] = (i2){tid, 9}; sreg[i] = (i2){tid, 3}; }
+  for (int i = 0; i < 2; i++) for (int j = 0; j < 4; j++) w[i][j] = __builtin_bit_cast(h8, (i4){tid, j, i, 7});
+#endif
+
+  // unpack the two words of 16-column group j2 of k step (slot, h) into w[buf]
+  auto dequant_pair = [&](int buf, int slot, int h, int j2) {
+#ifdef W4A16_PF_SKIP_DQ
+    return;
+#endif
+    h2 s2 = GROUP ? as_h2(sreg[slot][j2]) : (h2){(half_t)1.f, (half_t)1.f};
+    h2 l0, h0, l1, h1, m0_, n0_, m1_, n1_;
+    dequant_word<GROUP>(breg[slot][2 * h][j2], s2, dc, l0, h0, l1, h1);
+    dequant_word<GROUP>(breg[slot][2 * h + 1][j2], s2, dc, m0_, n0_, m1_, n1_);
+    w[buf][2 * j2] = make_h8(l0, h0, m0_, n0_);
+    w[buf][2 * j2 + 1] = make_h8(l1, h1, m1_, n1_);
+  };
+  auto read_frag = [&](int idx, const char* step_base, int i) {
+#ifdef W4A16_PF_SKIP_RD
+    return;
+#endif
+    af[idx] = *(const i4*)(step_base + a_rd + i * 256);
+  };
+
+  // One 32-deep k step: 32 MFMAs on w[h] and the operand ring, while the
+  // operands of the next step are fetched from LDS and its weights unpacked
+  // into w[h^1].  `mid` runs between the fourth and fifth row block.
+  auto step = [&](int h, const char* cur_base, const char* nxt_base, int nslot, int nh,
+                  auto&& mid) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      h8 af = __builtin_bit_cast(h8, *(const i4*)(base + i * 256));
+      if (i + 3 < 8)
+        read_frag((i + 3) & 3, cur_base, i + 3);
+      else
+        read_frag((i + 3) & 3, nxt_base, i + 3 - 8);
+      const h8 a = __builtin_bit_cast(h8, af[i & 3]);
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[j], af, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[h][j], a, acc[i][j], 0, 0, 0);
+      if (i == 1) dequant_pair(h ^ 1, nslot, nh, 0);
+      if (i == 3) mid();
+      if (i == 5) dequant_pair(h ^ 1, nslot, nh, 1);
     }
   };
 
-  // prologue: slab 0 -> LDS, slab 1 and the weights of stages 0, 1 in flight
+  // prologue: slab 0 in LDS, slab 1 and the weights of stages 0 and 1 in flight
   issue_a(0);
   issue_b(0, 0);
   store_a(0);
   issue_a(1);
   issue_b(1, 1);
+  dequant_pair(0, 0, 0, 0);
+  dequant_pair(0, 0, 0, 1);
   __syncthreads();
+  read_frag(0, smem, 0);
+  read_frag(1, smem, 1);
+  read_frag(2, smem, 2);
 
+  int ring = 0;  // LDS slab of the stage being computed
   for (int s = 0; s < stages; s += 2) {
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-      const int cs = s + u;  // stage being computed, slab in buffer u
-      step(u, u, 0);
-      store_a(u ^ 1);   // slab cs+1 (nobody reads that buffer during stage cs)
-      issue_a(cs + 2);
-      step(u, u, 1);
-      issue_b(u, cs + 2);
+      const int cs = s + u;
+      const int ring_next = ring == kPfRing - 1 ? 0 : ring + 1;
+      const char* cur = smem + ring * kPfStageBytes;
+      const char* nxt = smem + ring_next * kPfStageBytes;
+      // step 0: meanwhile slab cs+1 goes to LDS and slab cs+2 is requested.
+      // The slab written here was last read two stages ago, and every wave
+      // has passed the previous barrier since, so one barrier per stage is
+      // enough; it sits mid-stage, where no wave needs the new slab yet.
+      step(0, cur, cur + kPfStepBytes, u, 1, [&]() {
+        store_a(ring_next);
+        issue_a(cs + 2);
+      });
       __syncthreads();
+      // step 1: the weights of this stage are spent, request stage cs+2
+      step(1, cur + kPfStepBytes, nxt, u ^ 1, 0, [&]() { issue_b(u, cs + 2); });
+      ring = ring_next;
     }
   }
+
+  // add the second k half to the first through LDS, four row blocks at a time
+  // (4 waves x 16 KiB per round; the slab rings are dead by now)
+#pragma unroll
+  for (int r = 0; r < 2; r++) {
+    __syncthreads();
+    f4* ex = (f4*)smem_all + (size_t)wave * (16 * 64);
+    if (kh == 1) {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) ex[(i * 4 + j) * 64 + lane] = acc[4 * r + i][j];
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[4 * r + i][j] += ex[(i * 4 + j) * 64 + lane];
+    }
+  }
+  if (kh == 1) return;
 
   // epilogue: lane holds row m = 16 i + nu and, per (j2, h), four consecutive columns
   half_t* C = (half_t*)p.C;
@@ -189,11 +286,22 @@ int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream) {
   const int tiles_m = ceil_div(a.M, kPfTileM);
   const int tiles_n = a.N / kPfTileN;
   const int grid = tiles_m * tiles_n;
+  // more LDS than the default per-workgroup limit: opt in once per kernel
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)prefill_kernel<true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)prefill_kernel<false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess)
+      return 3;
+    configured = true;
+  }
   if (group)
-    hipLaunchKernelGGL(prefill_kernel<true>, dim3(grid), dim3(256), 0, stream, a, tiles_m, tiles_n);
+    hipLaunchKernelGGL(prefill_kernel<true>, dim3(grid), dim3(512), kPfLdsBytes, stream, a,
+                       tiles_m, tiles_n);
   else
-    hipLaunchKernelGGL(prefill_kernel<false>, dim3(grid), dim3(256), 0, stream, a, tiles_m,
-                       tiles_n);
+    hipLaunchKernelGGL(prefill_kernel<false>, dim3(grid), dim3(512), kPfLdsBytes, stream, a,
+                       tiles_m, tiles_n);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
