@@ -28,6 +28,16 @@
 #ifndef W4A16_PF_K
 #define W4A16_PF_K(s) (s)
 #endif
+#ifndef W4A16_PF_T0
+#define W4A16_PF_T0
+#define W4A16_PF_T1
+#define W4A16_PF_TBEGIN
+#define W4A16_PF_TEND
+#endif
+#ifndef W4A16_PF_TENTRY
+#define W4A16_PF_TENTRY
+#define W4A16_PF_TEXIT
+#endif
 
 namespace w4a16 {
 
@@ -36,8 +46,10 @@ namespace {
 constexpr int kPfTileM = 128;
 constexpr int kPfTileN = 256;
 constexpr int kPfStageK = 64;
-constexpr int kPfStepBytes = 4 * 128 * 16 + 128;  // one 32-deep k step of the slab (+pad)
-constexpr int kPfStageBytes = 2 * kPfStepBytes;   // two steps per stage
+constexpr int kPfStepBytes = 4 * 128 * 16 + 128;  // one 32-deep k step of the A slab (+pad)
+constexpr int kPfSlabA = 2 * kPfStepBytes;        // two steps per stage
+constexpr int kPfSlabB = 4 * 2048;                // four 16-deep rows of packed weights
+constexpr int kPfStageBytes = kPfSlabA + kPfSlabB;
 constexpr int kPfRing = 3;                        // slabs in LDS per k half
 constexpr int kPfLdsBytes = 2 * kPfRing * kPfStageBytes;
 constexpr int kOobPf = (int)0x80000000;
@@ -51,6 +63,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigne
 template <bool GROUP>
 __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) char smem_all[];  // kPfLdsBytes
+  W4A16_PF_TENTRY
 
   const int kh = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);  // k half
   const int tid = threadIdx.x & 255;  // thread within the half
@@ -80,7 +93,17 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       pf_rsrc((const char*)p.A + (size_t)m0 * p.K * 2, (unsigned)rows * (unsigned)p.K * 2u);
   const int b_row = p.N * 8;
 
-  const int b_lane = 1024 * (2 * tn + pr) + 64 * nu + 16 * kg + 8 * jp;
+  // Packed weights go through LDS too: the 256 threads of a half copy the
+  // stage's four 2 KiB rows with coalesced 16-byte loads, and every lane then
+  // picks its 8 bytes (Marlin piece (t = kg, c = nu%8) of block 2p + nu/8,
+  // words 2jp, 2jp+1).  Pieces are rotated inside each group of four so that
+  // those reads are free of bank conflicts.
+  const int bx = tid & 127;  // 16-byte piece inside a row, for the copy
+  const int b_ld = 2048 * tn + 16 * bx;
+  const int b_a = (bx & 63) >> 2;
+  const int b_wr = kPfSlabA + (wave >> 1) * 2048 + (bx >> 6) * 1024 +
+                   16 * (4 * b_a + (((bx & 3) + (b_a >> 2)) & 3));
+  const int b_rd = kPfSlabA + pr * 1024 + 16 * (4 * nu + ((kg + (nu >> 2)) & 3)) + 8 * jp;
   const int s_lane = (256 * tn + 128 * pr + 8 * nu) * 2 + 8 * jp;
 
   // slab staging: thread (row = tid/8 + 32 i, chunk x = tid%8) moves 16 bytes;
@@ -105,43 +128,43 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   const int s_end = kh ? stages_all : half_stages;
   const int stages = half_stages;
 
-  i4 areg[4];     // slab of the stage after next, in flight
-  i2 breg[2][4];  // weight words of two stages: 4 rows x 8 bytes each
-  i2 sreg[2];
+  i4 areg[4];   // A slab of the stage after next, in flight
+  i4 bcopy[2];  // its packed weights
+  i2 sreg[2];   // group scales of this stage and the next
 
-  auto issue_b = [&](int slot, int s) {
-#ifdef W4A16_PF_SKIP_B
-    return;
-#endif
+  auto issue_s = [&](int slot, int s) {
     const int sg = s_begin + s;  // stage in the whole k range
     const int inv = sg < s_end ? 0 : kOobPf;
-#pragma unroll
-    for (int r = 0; r < 4; r++)
-      breg[slot][r] = __builtin_amdgcn_raw_buffer_load_b64(rB, b_lane | inv,
-                                                           (4 * W4A16_PF_K(sg) + r) * b_row, 0);
     if (GROUP)
       sreg[slot] = __builtin_amdgcn_raw_buffer_load_b64(rS, s_lane | inv,
                                                         (W4A16_PF_K(sg) >> 1) * p.N * 2, 0);
   };
   auto issue_a = [&](int s) {
-#ifdef W4A16_PF_SKIP_A
-    return;
-#endif
     const int sg = s_begin + s;
     const int inv = sg < s_end ? 0 : kOobPf;
+#ifndef W4A16_PF_SKIP_A
 #pragma unroll
     for (int i = 0; i < 4; i++)
       areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
+#endif
+#ifndef W4A16_PF_SKIP_B
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      bcopy[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          rB, b_ld | inv, (4 * W4A16_PF_K(sg) + 2 * i + (wave >> 1)) * b_row, 0);
+#endif
   };
   auto store_a = [&](int ring) {
 #ifdef W4A16_PF_SKIP_ST
     return;
 #endif
-    char* base = smem + ring * kPfStageBytes + a_wr;
+    char* base = smem + ring * kPfStageBytes;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-      for (int g = 0; g < 4; g++) *(int*)(base + g * 2048 + i * 32 * 16) = areg[i][g];
+      for (int g = 0; g < 4; g++) *(int*)(base + a_wr + g * 2048 + i * 32 * 16) = areg[i][g];
+#pragma unroll
+    for (int i = 0; i < 2; i++) *(i4*)(base + b_wr + i * 4096) = bcopy[i];
   };
 
   f4 acc[8][4];
@@ -152,9 +175,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 
   h8 w[2][4];  // unpacked weights of the current and the next k step
   i4 af[4];    // ring of activation operands, three ahead of the MFMAs
+  i2 bw[2];    // packed weight words of the next k step (its two 16-deep rows)
 #ifdef W4A16_PF_INIT
   for (int i = 0; i < 4; i++) { areg[i] = (i4){tid, 1, 2, 3}; af[i] = (i4){tid, 5, 6, 7}; }
-  for (int i = 0; i < 2; i++) for (int r = 0; r < 4; r++) { breg[i][r] = (i2){tid, 9}; sreg[i] = (i2){tid, 3}; }
+  for (int i = 0; i < 2; i++) { bcopy[i] = (i4){tid, 9, 1, 2}; sreg[i] = (i2){tid, 3}; }
   for (int i = 0; i < 2; i++) for (int j = 0; j < 4; j++) w[i][j] = __builtin_bit_cast(h8, (i4){tid, j, i, 7});
 #endif
 
@@ -163,12 +187,21 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #ifdef W4A16_PF_SKIP_DQ
     return;
 #endif
+    (void)h;
     h2 s2 = GROUP ? as_h2(sreg[slot][j2]) : (h2){(half_t)1.f, (half_t)1.f};
     h2 l0, h0, l1, h1, m0_, n0_, m1_, n1_;
-    dequant_word<GROUP>(breg[slot][2 * h][j2], s2, dc, l0, h0, l1, h1);
-    dequant_word<GROUP>(breg[slot][2 * h + 1][j2], s2, dc, m0_, n0_, m1_, n1_);
+    dequant_word<GROUP>(bw[0][j2], s2, dc, l0, h0, l1, h1);
+    dequant_word<GROUP>(bw[1][j2], s2, dc, m0_, n0_, m1_, n1_);
     w[buf][2 * j2] = make_h8(l0, h0, m0_, n0_);
     w[buf][2 * j2 + 1] = make_h8(l1, h1, m1_, n1_);
+  };
+  // fetch the packed words of k step h of the slab at `stage_base`
+  auto read_bw = [&](const char* stage_base, int h) {
+#ifdef W4A16_PF_SKIP_RD
+    return;
+#endif
+    bw[0] = *(const i2*)(stage_base + b_rd + (2 * h) * 2048);
+    bw[1] = *(const i2*)(stage_base + b_rd + (2 * h + 1) * 2048);
   };
   auto read_frag = [&](int idx, const char* step_base, int i) {
 #ifdef W4A16_PF_SKIP_RD
@@ -180,10 +213,11 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // One 32-deep k step: 32 MFMAs on w[h] and the operand ring, while the
   // operands of the next step are fetched from LDS and its weights unpacked
   // into w[h^1].  `mid` runs between the fourth and fifth row block.
-  auto step = [&](int h, const char* cur_base, const char* nxt_base, int nslot, int nh,
-                  auto&& mid) {
+  auto step = [&](int h, const char* cur_base, const char* nxt_base, const char* nxt_stage,
+                  int nslot, int nh, auto&& mid) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
+      if (i == 0) read_bw(nxt_stage, nh);
       if (i + 3 < 8)
         read_frag((i + 3) & 3, cur_base, i + 3);
       else
@@ -192,26 +226,28 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
       for (int j = 0; j < 4; j++)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[h][j], a, acc[i][j], 0, 0, 0);
-      if (i == 1) dequant_pair(h ^ 1, nslot, nh, 0);
+      if (i == 2) dequant_pair(h ^ 1, nslot, nh, 0);
       if (i == 3) mid();
       if (i == 5) dequant_pair(h ^ 1, nslot, nh, 1);
     }
   };
 
-  // prologue: slab 0 in LDS, slab 1 and the weights of stages 0 and 1 in flight
+  // prologue: slab 0 in LDS, slab 1 in flight, scales of stages 0 and 1
   issue_a(0);
-  issue_b(0, 0);
+  issue_s(0, 0);
+  issue_s(1, 1);
   store_a(0);
   issue_a(1);
-  issue_b(1, 1);
+  __syncthreads();
+  read_bw(smem, 0);
   dequant_pair(0, 0, 0, 0);
   dequant_pair(0, 0, 0, 1);
-  __syncthreads();
   read_frag(0, smem, 0);
   read_frag(1, smem, 1);
   read_frag(2, smem, 2);
 
   int ring = 0;  // LDS slab of the stage being computed
+  W4A16_PF_TBEGIN
   for (int s = 0; s < stages; s += 2) {
 #pragma unroll
     for (int u = 0; u < 2; u++) {
@@ -223,63 +259,82 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       // The slab written here was last read two stages ago, and every wave
       // has passed the previous barrier since, so one barrier per stage is
       // enough; it sits mid-stage, where no wave needs the new slab yet.
-      step(0, cur, cur + kPfStepBytes, u, 1, [&]() {
+      step(0, cur, cur + kPfStepBytes, cur, u, 1, [&]() {
         store_a(ring_next);
         issue_a(cs + 2);
       });
+      W4A16_PF_T0
       __syncthreads();
-      // step 1: the weights of this stage are spent, request stage cs+2
-      step(1, cur + kPfStepBytes, nxt, u ^ 1, 0, [&]() { issue_b(u, cs + 2); });
+      W4A16_PF_T1
+      // step 1: the scales of this stage are spent, request those of stage cs+2
+      step(1, cur + kPfStepBytes, nxt, nxt, u ^ 1, 0, [&]() {});
+      issue_s(u, cs + 2);
       ring = ring_next;
     }
   }
 
-  // add the second k half to the first through LDS, four row blocks at a time
-  // (4 waves x 16 KiB per round; the slab rings are dead by now)
+  W4A16_PF_TEND
+  // ---- epilogue.  The k halves swap the row blocks they will not write
+  // (half 0 keeps blocks 0-3, half 1 keeps 4-7) through LDS and add; the slab
+  // rings are dead by now.
+  const int own = 4 * kh;  // first row block this wave finishes
+  __syncthreads();
+  {
+    f4* out = (f4*)smem_all + (size_t)(kh * 4 + wave) * (16 * 64);
 #pragma unroll
-  for (int r = 0; r < 2; r++) {
-    __syncthreads();
-    f4* ex = (f4*)smem_all + (size_t)wave * (16 * 64);
-    if (kh == 1) {
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-      for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) ex[(i * 4 + j) * 64 + lane] = acc[4 * r + i][j];
-    }
-    __syncthreads();
-    if (kh == 0) {
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[4 * r + i][j] += ex[(i * 4 + j) * 64 + lane];
-    }
+      for (int j = 0; j < 4; j++)
+        out[(i * 4 + j) * 64 + lane] = kh ? acc[i][j] : acc[4 + i][j];
   }
-  if (kh == 1) return;
+  __syncthreads();
+  f4 fin[4][4];
+  {
+    const f4* in = (const f4*)smem_all + (size_t)((kh ^ 1) * 4 + wave) * (16 * 64);
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        fin[i][j] = (kh ? acc[4 + i][j] : acc[i][j]) + in[(i * 4 + j) * 64 + lane];
+  }
+  __syncthreads();
 
-  // epilogue: lane holds row m = 16 i + nu and, per (j2, h), four consecutive columns
-  half_t* C = (half_t*)p.C;
+  // fp16 tile -> LDS in row-major order, then whole 512-byte rows go out with
+  // coalesced 16-byte stores.  Lane holds row 16 i + nu and, per (j2, h), four
+  // consecutive columns.
+  constexpr int kPitch = kPfTileN * 2 + 16;  // bytes per tile row in LDS
   const int q = lane >> 4;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
-    const int n0 = kPfTileN * tn + 128 * pr + 64 * (q >> 1) + 16 * (2 * jp + (j >> 1)) +
-                   8 * (j & 1) + 4 * (q & 1);
+    const int nloc = 128 * pr + 64 * (q >> 1) + 16 * (2 * jp + (j >> 1)) + 8 * (j & 1) + 4 * (q & 1);
     h4 sc = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
     if (!GROUP) {
       const half_t* S = (const half_t*)p.S;
 #pragma unroll
-      for (int r = 0; r < 4; r++) sc[r] = S[scale_index_single(n0 + r)];
+      for (int r = 0; r < 4; r++) sc[r] = S[scale_index_single(kPfTileN * tn + nloc + r)];
     }
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int m = 16 * i + nu;
-      if (m < rows) {
-        h4 o = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2],
-                (half_t)acc[i][j][3]};
-        if (!GROUP) o *= sc;
-        *(h4*)(C + (size_t)(m0 + m) * p.N + n0) = o;
-      }
+    for (int i = 0; i < 4; i++) {
+      const int m = 16 * (own + i) + nu;
+      h4 o = {(half_t)fin[i][j][0], (half_t)fin[i][j][1], (half_t)fin[i][j][2],
+              (half_t)fin[i][j][3]};
+      if (!GROUP) o *= sc;
+      *(h4*)(smem_all + m * kPitch + nloc * 2) = o;
     }
   }
+  __syncthreads();
+  half_t* C = (half_t*)p.C;
+#pragma unroll
+  for (int it = 0; it < 8; it++) {
+    const int piece = it * 512 + (int)threadIdx.x;  // 16-byte piece of the tile
+    const int m = piece >> 5;
+    const int c16 = piece & 31;
+    if (m < rows) {
+      const i4 v = *(const i4*)(smem_all + m * kPitch + c16 * 16);
+      *(i4*)(C + (size_t)(m0 + m) * p.N + kPfTileN * tn + c16 * 8) = v;
+    }
+  }
+  W4A16_PF_TEXIT
 }
 
 int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream) {
