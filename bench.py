@@ -170,6 +170,9 @@ def main():
     ap.add_argument("--shape", default="headline",
                     help="headline (decode + batch16 + prefill) or one of: " + ", ".join(SHAPES))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 "
@@ -192,6 +195,14 @@ def main():
         gflop = 2.0 * M * N * K / 1e9
         cap = 2000 if gflop < 2 else (400 if gflop < 40 else 100)
         return max(1, min(args.steps, cap)) if name != main_name else args.steps
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup)
     shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup) for n in others]

@@ -1,0 +1,226 @@
+"""CPU-only tests of the host side: the C ABI library loads and exports what
+include/marlin_amd.h declares, the argument contract matches the reference
+launcher's return codes, the stream-K partition covers every granule exactly
+once, and the Python mirror of the reference's `marlin` module packs the way
+the oracle does.  No GPU work is launched here.
+"""
+import ctypes
+import os
+import re
+import sys
+
+import numpy as np
+import pytest
+
+import _oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
+LIB = os.path.join(ROOT, "awesome-cute_amd", "libmarlin_amd.so")
+
+
+@pytest.fixture(scope="module")
+def marlin():
+    if not os.path.exists(LIB):
+        pytest.fail("libmarlin_amd.so is not built; run `python __graft_entry__.py build`")
+    import marlin as m
+    return m
+
+
+def test_library_exports_every_declared_symbol(marlin):
+    header = open(os.path.join(ROOT, "include", "marlin_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = re.findall(r"\b(marlin_\w+)\s*\(", header)
+    assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
+            "marlin_amd_plan", "marlin_amd_last_error", "marlin_amd_version"} <= set(names)
+    lib = ctypes.CDLL(LIB)
+    for n in set(names):
+        assert hasattr(lib, n), n
+    assert b"gfx950" in marlin._lib.marlin_amd_version()
+
+
+def test_oracle_is_not_linked_into_the_product():
+    out = os.popen(f"ldd {LIB}").read()
+    assert "w4a16_ref" not in out
+    src = os.path.join(ROOT, "awesome-cute_amd")
+    for dirpath, _, files in os.walk(src):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text.lower() or f == "build.py", (dirpath, f)
+
+
+# return codes of the reference launcher (marlin_cute_kernel.cu:39-60,95-107)
+@pytest.mark.parametrize("args,want", [
+    ((16, 256, 512, 128, -1, -1), 0),      # BASELINE config 1
+    ((1, 4096, 4096, 128, -1, -1), 0),
+    ((2048, 4096, 4096, 128, -1, -1), 0),
+    ((64, 28672, 8192, -1, -1, -1), 0),
+    ((0, 256, 512, 128, -1, -1), 0),       # empty problem is fine
+    ((16, 0, 512, -1, -1, -1), 0),
+    ((16, 256, 64, -1, 128, 128), 1),      # marlin_test.py:105 (k=64, thread_k=128)
+    ((16, 256, 64, -1, 256, 256), 1),      # marlin_test.py:111
+    ((16, 256, 64, 32, 256, 256), 1),      # marlin_test.py:118 (shape check comes first)
+    ((16, 256, 64, 32, 64, 256), 2),       # groupsize 32: no kernel
+    ((16, 128, 512, 128, -1, -1), 0),      # n=128 only with the small tile
+    ((17, 128, 512, 128, -1, -1), 1),      # auto tile is (64,256) above 16 rows
+    ((32, 256, 512, 128, 128, 128), 2),    # small tile has no kernel for 32 rows
+    ((16, 256, 512, 128, 64, 128), 2),     # unknown tile
+    ((16, 256, 192, -1, 64, 256), 0),      # marlin_test.py:93 (k=192, per-channel)
+    ((16, 256, 192, 128, 64, 256), 1),     # k not a multiple of the group
+    ((16, 256, 512, 128, 0, 128), 1),
+    ((16, 256, 512, 0, -1, -1), 2),
+])
+def test_shape_contract(marlin, args, want):
+    assert marlin.check(*args) == want
+
+
+def test_binding_level_errors_without_gpu(marlin):
+    """marlin_mul rejects bad group counts and short workspaces before any
+    device work (marlin_gemm.cpp:27-31); null pointers are never touched."""
+    err = ctypes.create_string_buffer(256)
+    f = marlin._lib.marlin_mul
+    rc = f(None, None, None, None, 16, 256, 64, 3, None, 32, 0, None, -1, -1, -1, 16, 1, err, 256)
+    assert rc == 4 and b"not compatible with 3 groups" in err.value
+    rc = f(None, None, None, None, 16, 256, 64, 1, None, 2, 0, None, 128, 128, -1, 16, 1, err, 256)
+    assert rc == 5 and b"workspace must be of size at least 32" in err.value
+    rc = f(None, None, None, None, 16, 256, 64, 1, None, 32, 0, None, 128, 128, -1, 16, 1, err, 256)
+    assert rc == 1 and b"thread_k=128" in err.value
+    rc = f(None, None, None, None, 16, 256, 64, 2, None, 32, 0, None, 64, 256, -1, 16, 1, err, 256)
+    assert rc == 2 and b"groupsize=32" in err.value
+    # an empty problem is accepted and does nothing
+    rc = f(None, None, None, None, 0, 256, 128, 1, None, 32, 0, None, -1, -1, -1, 16, 1, err, 256)
+    assert rc == 0
+
+
+def _partition(plan):
+    """Re-derivation of the stream-K ownership from the plan's four numbers."""
+    NT, KG, gpb, grid = (plan[k] for k in ("col_tiles", "granules_per_tile",
+                                           "granules_per_wg", "grid"))
+    total = NT * KG
+    owner = np.full(total, -1)
+    for b in range(grid):
+        lo, hi = b * gpb, min(total, (b + 1) * gpb)
+        assert lo < hi, "every launched workgroup owns at least one granule"
+        assert (owner[lo:hi] == -1).all()
+        owner[lo:hi] = b
+    assert (owner >= 0).all(), "every granule has exactly one owner"
+    return owner.reshape(NT, KG)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192),
+                                 (128, 128), (256, 192), (512, 1024), (1280, 1152)])
+@pytest.mark.parametrize("sms", [1, 2, 3, 7, 31, 100, 255, 256, 304, 512, 1024, 5000])
+def test_stream_partition_properties(marlin, n, k, sms):
+    m = 16 if n % 256 else 48
+    rc, plan = marlin.plan(m, n, k, -1, -1, -1, sms, 256)
+    assert rc == 0 and plan["kernel"] == 1
+    assert plan["grid"] <= min(max(sms, 1), 1024)
+    owner = _partition(plan)
+    gpb = plan["granules_per_wg"]
+    slots = set()
+    for t in range(owner.shape[0]):
+        sharers = sorted(set(owner[t].tolist()))
+        # contributors of a tile are consecutive workgroups
+        assert sharers == list(range(sharers[0], sharers[-1] + 1))
+        assert sharers[0] == (t * owner.shape[1]) // gpb
+        assert sharers[-1] == ((t + 1) * owner.shape[1] - 1) // gpb
+        if len(sharers) > 1:
+            for b in sharers:
+                first_tile = (b * gpb) // owner.shape[1]
+                slot = 2 * b + (1 if t != first_tile else 0)
+                assert slot not in slots, "partial-sum slots never collide"
+                slots.add(slot)
+    # a workgroup shares at most its first and its last tile
+    for b in range(plan["grid"]):
+        tiles = np.unique(np.nonzero(owner == b)[0])
+        for t in tiles[1:-1]:
+            assert (owner[t] == b).all()
+
+
+def test_plan_picks_kernels(marlin):
+    assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 1
+    assert marlin.plan(64, 28672, 8192, 128)[1]["kernel"] == 1
+    rc, p = marlin.plan(2048, 4096, 4096, 128)
+    assert rc == 0 and p["kernel"] == 2 and p["grid"] == 16 * 16
+    assert marlin.plan(16, 256, 64, -1, 128, 128)[0] == 1
+
+
+# ------------------------------------------------------------ Python mirror
+
+def test_perms_match_oracle(marlin):
+    perm, sp, sps = O.get_perms()
+    assert np.array_equal(marlin._perm.numpy(), perm)
+    assert marlin._scale_perm == sp.tolist()
+    assert marlin._scale_perm_single == sps.tolist()
+
+
+@pytest.mark.parametrize("k,n", [(16, 64), (128, 256), (512, 768)])
+def test_pack_weights_matches_oracle(marlin, k, n):
+    import torch
+    q = np.random.default_rng(k + n).integers(0, 16, (k, n), dtype=np.uint8)
+    B = marlin.pack_weights(torch.from_numpy(q.astype(np.int32)))
+    assert B.dtype == torch.int32
+    assert np.array_equal(B.numpy(), O.pack_weights(q))
+
+
+@pytest.mark.parametrize("groupwise", [True, False])
+def test_pack_scales_matches_oracle(marlin, groupwise):
+    import torch
+    s = np.random.default_rng(7).uniform(0.001, 0.02, (4 if groupwise else 1, 512)).astype(np.float16)
+    got = marlin.pack_scales(torch.from_numpy(s), groupwise).numpy()
+    assert np.array_equal(got.view(np.uint16), O.pack_scales(s, groupwise).view(np.uint16))
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_layer_pack_on_cpu(marlin, groupsize):
+    """Layer.pack (marlin.py:92-131) from a fake-quantised Linear: the packed
+    buffers decode back to the quantiser's integers and scales."""
+    import torch
+    k, n = 256, 256
+    w = np.random.default_rng(3).standard_normal((k, n)).astype(np.float16)
+    q, s, ref = O.gen_quant4(w, groupsize)
+    linear = torch.nn.Linear(k, n, bias=False)
+    linear.weight.data = torch.from_numpy(ref).t().contiguous()
+    layer = marlin.Layer(k, n, groupsize=groupsize)
+    layer.pack(linear, torch.from_numpy(s).t().contiguous())
+    assert np.array_equal(O.unpack_weights(layer.B.numpy(), k, n), q)
+    assert np.array_equal(O.unpack_scales(layer.s.numpy(), groupsize != -1).view(np.uint16),
+                          s.view(np.uint16))
+    assert layer.workspace.numel() == n // 128 * 16 and not layer.workspace.any()
+
+
+def test_quantize_matches_oracle_quantiser(marlin):
+    import torch
+    w = np.random.default_rng(5).standard_normal((256, 128)).astype(np.float16)
+    for g in (128, -1):
+        ref, q, s = marlin.quantize(torch.from_numpy(w), g)
+        q0, s0, ref0 = O.gen_quant4(w, g)
+        assert np.array_equal(q.numpy(), q0)
+        assert np.array_equal(s.numpy().view(np.uint16), s0.view(np.uint16))
+        assert np.array_equal(ref.numpy().view(np.uint16), ref0.view(np.uint16))
+
+
+def test_layer_rejects_what_the_reference_rejects(marlin):
+    with pytest.raises(ValueError):
+        marlin.Layer(256, 256, groupsize=64)
+    with pytest.raises(ValueError):
+        marlin.Layer(192, 256)
+    with pytest.raises(ValueError):
+        marlin.Layer(256, 128)
+
+
+def test_replace_linear(marlin):
+    import torch.nn as nn
+    model = nn.Sequential(nn.Linear(256, 512), nn.ReLU(), nn.Sequential(nn.Linear(512, 256)))
+    marlin.replace_linear(model, groupsize=128)
+    assert isinstance(model[0], marlin.Layer) and isinstance(model[2][0], marlin.Layer)
+    assert model[0].k == 256 and model[0].n == 512 and model[0].groupsize == 128
+    marlin.replace_linear(model)  # Layers are left alone
+
+
+def test_mul_refuses_cpu_tensors(marlin):
+    import torch
+    A = torch.zeros((1, 128), dtype=torch.half)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        marlin.mul(A, A, A, A, A)
