@@ -39,9 +39,14 @@ SHAPES = {
     "large_chan": (64, 28672, 8192, -1, "hbm"),
 }
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (see profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE and scaled by what the same counters read for a 256 MiB device copy
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this pool); the summaries are under
+# profiles/.  None for workloads not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "decode": int((4979.9 * 2.0 + 2375.1) * 1024),
+    "prefill": int((42060.6 * 2.0 + 16384.0) * 1024),
+}
 
 
 def build_inputs(torch, O, M, N, K, groupsize, nbuf, seed=0):
