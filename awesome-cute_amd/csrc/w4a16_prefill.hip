@@ -246,6 +246,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   read_frag(1, smem, 1);
   read_frag(2, smem, 2);
 
+  // The instruction arbiter favours the older waves (the first k half), which
+  // then idle at every barrier; a higher priority for the second half evens
+  // the two out (measured: 4 % faster).
+  if (kh) __builtin_amdgcn_s_setprio(1);
   int ring = 0;  // LDS slab of the stage being computed
   W4A16_PF_TBEGIN
   for (int s = 0; s < stages; s += 2) {
