@@ -128,9 +128,39 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
     return pl;
   }
   pl.kernel = 1;
-  int want = sms > 0 ? sms : cus * env_int("MARLIN_AMD_STREAM_WG_PER_CU", 1);
-  if (want > kMaxStreamGrid) want = kMaxStreamGrid;
-  pl.sp = make_stream_plan(n, k, want);
+  if (sms > 0) {
+    pl.sp = make_stream_plan(n, k, sms > kMaxStreamGrid ? kMaxStreamGrid : sms);
+  } else {
+    // Granules per workgroup.  Measured on MI355X: a split that cuts column
+    // tiles at whole fractions (or multiples) of a tile costs about
+    // 0.1 us x row blocks per granule of the longest workgroup; a split that
+    // leaves workgroups straddling tile boundaries pays for a second fix-up
+    // per workgroup, about 1 + 2.5 x row blocks us on top.  Take the cheapest
+    // of the aligned candidates and the evenly balanced one.
+    const int mb = ceil_div(m < kStreamMaxRows ? m : kStreamMaxRows, 16);
+    const int KG = k / kGranuleK;
+    const int total = (n / kTileN) * KG;
+    const double per_granule = 0.1 * mb, straddle = 1.0 + 2.5 * mb;
+    int best = ceil_div(total, cus);
+    double best_cost = per_granule * best + ((best % KG == 0 || KG % best == 0) ? 0.0 : straddle);
+    auto consider = [&](int g) {
+      if (g < 1 || g > total) return;
+      const int grid = ceil_div(total, g);
+      if (grid > cus) return;  // more workgroups than CUs never paid off
+      const double cost = per_granule * g;
+      if (cost < best_cost - 1e-9 || (cost < best_cost + 1e-9 && g > best)) {
+        best = g;
+        best_cost = cost;
+      }
+    };
+    for (int d = 1; d <= KG; d++)
+      if (KG % d == 0) consider(KG / d);
+    for (int mult = 2; mult * KG <= total; mult++) consider(mult * KG);
+    pl.sp.NT = n / kTileN;
+    pl.sp.KG = KG;
+    pl.sp.gpb = best;
+    pl.sp.grid = ceil_div(total, best);
+  }
   pl.grid = pl.sp.grid;
   pl.launches = ceil_div(m, kStreamMaxRows);
   return pl;
