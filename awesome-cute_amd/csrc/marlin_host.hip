@@ -168,7 +168,12 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
 
 int run(const void* A, const void* B, void* C, const void* s, int m, int n, int k,
         void* workspace, int groupsize, int dev, hipStream_t stream, int thread_k, int thread_n,
-        int sms) {
+        int sms, int max_par) {
+  // the caller's workspace holds at least n/128 * max_par zero ints
+  // (reference marlin_gemm.cpp:29-31, marlin_cute_kernel.cu:68); one counter
+  // per column tile is used, and the counters are spread max_par ints apart
+  // (64 bytes at the launcher's default of 16)
+  const int lock_stride = max_par < 1 ? 1 : (max_par > 16 ? 16 : max_par);
   int rc = check_shape(m, n, k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || m == 0 || n == 0 || k == 0) return rc;
   if (dev < 0 || dev >= kMaxDevices) {
@@ -200,6 +205,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
       a.N = n;
       a.K = k;
       a.locks = (int*)workspace;
+      a.lock_stride = lock_stride;
       a.scratch = nullptr;
       a.gpb = 0;
       rc = launch_prefill(a, groupsize != -1, stream);
@@ -216,6 +222,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
         a.N = n;
         a.K = k;
         a.locks = (int*)workspace;
+        a.lock_stride = lock_stride;
         a.scratch = scratch;
         a.gpb = pl.sp.gpb;
         rc = launch_stream(a, groupsize != -1, pl.grid, stream);
@@ -234,9 +241,8 @@ extern "C" {
 int marlin_gemm(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n,
                 int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k,
                 int thread_n, int sms, int max_par) {
-  (void)max_par;
   return run(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, (hipStream_t)stream,
-             thread_k, thread_n, sms);
+             thread_k, thread_n, sms, max_par);
 }
 
 int marlin_cute(const void* A, const void* B, void* C, void* s, int prob_m, int prob_n,

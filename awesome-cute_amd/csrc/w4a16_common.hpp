@@ -95,8 +95,8 @@ __device__ __forceinline__ unsigned pack_half2(float a, float b) {
 
 // ---------------------------------------------------------------------------
 // Stream-K partition of the streaming kernel.  The work of one launch is the
-// linear space of NT * KG granules (column tile major, k minor); workgroup b
-// owns granules [b*gpb, (b+1)*gpb).  A column tile whose granules fall into
+// linear space of NT * KG granules (column tile major, k minor); the workgroup
+// with work index b owns granules [b*gpb, (b+1)*gpb).  A column tile whose granules fall into
 // more than one workgroup is finished by whichever of them arrives last at the
 // tile's counter.
 struct StreamPlan {
@@ -120,7 +120,27 @@ __host__ __device__ inline StreamPlan make_stream_plan(int N, int K, int want_gr
   return p;
 }
 
-// first / last workgroup touching tile t
+// The hardware deals workgroups to the 8 XCDs round-robin (blockIdx % 8) and
+// every XCD has an L2 of its own.  Workgroup blockIdx takes the work index
+// below, so that consecutive work indices (the sharers of a column tile) sit
+// behind one L2.  This is a placement hint only: the kernel checks the XCD it
+// really runs on before it trusts a line of that L2.
+__host__ __device__ __forceinline__ int xcd_work_index(int block, int grid) {
+  const int x = block & 7, q = grid >> 3, rem = grid & 7;
+  return x * q + (x < rem ? x : rem) + (block >> 3);
+}
+// True if `block` runs on the XCD the round-robin dealing predicts (xcd is
+// the one it really runs on) and that XCD's run of work indices holds all of
+// [first, last].
+__host__ __device__ __forceinline__ bool xcd_range_holds(int block, int grid, int xcd, int first,
+                                                         int last) {
+  const int x = block & 7, q = grid >> 3, rem = grid & 7;
+  const int lo = x * q + (x < rem ? x : rem);
+  const int hi = lo + q + (x < rem ? 1 : 0);
+  return xcd == x && first >= lo && last < hi;
+}
+
+// first / last workgroup (by work index) touching tile t
 __host__ __device__ __forceinline__ int tile_first_block(const StreamPlan& p, int t) {
   return (t * p.KG) / p.gpb;
 }
@@ -131,8 +151,8 @@ __host__ __device__ __forceinline__ int tile_last_block(const StreamPlan& p, int
 // Every workgroup owns at most two tiles that it shares with others (its
 // first and its last); a shared tile's partial sums go to slot 2b or 2b+1.
 __host__ __device__ __forceinline__ int partial_slot(const StreamPlan& p, int block, int t) {
-  int first_tile = (block * p.gpb) / p.KG;
-  return 2 * block + (t != first_tile ? 1 : 0);
+  // block touches tile t; t is its first tile unless the block starts before it
+  return 2 * block + (block * p.gpb < t * p.KG ? 1 : 0);
 }
 
 struct GemmArgs {
@@ -141,13 +161,17 @@ struct GemmArgs {
   void* C;          // (M, N) fp16 row-major
   const void* S;    // (K/128, N) or (1, N) fp16, Marlin-permuted
   int M, N, K;
-  int* locks;       // >= N/128 ints, zero on entry, zero on exit
+  int* locks;       // N/128 counters, lock_stride ints apart; zero on entry and on exit
+  int lock_stride;  // >= 1; spreads the counters over separate cache lines
   float* scratch;   // partial sums of shared tiles
   int gpb;          // granules per workgroup (streaming kernel)
 };
 
-// bytes of fp32 partial sums one slot holds for mb row blocks of 16
-constexpr size_t stream_slot_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
+// bytes of fp32 partial sums of mb row blocks of 16; a slot holds them twice
+// (a write-back copy for readers behind the same L2, a write-through copy for
+// everybody else)
+constexpr size_t stream_partial_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
+constexpr size_t stream_slot_bytes(int mb) { return 2 * stream_partial_bytes(mb); }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream);

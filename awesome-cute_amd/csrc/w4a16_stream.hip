@@ -25,6 +25,12 @@
 #define W4A16_STAMP_DECL
 #define W4A16_STAMP(i)
 #endif
+#ifndef W4A16_NOTE
+#define W4A16_NOTE(i, v)
+#endif
+#ifndef W4A16_COMPUTE_REPS
+#define W4A16_COMPUTE_REPS 1
+#endif
 
 namespace w4a16 {
 
@@ -48,6 +54,15 @@ __device__ __forceinline__ void store_device_scope(f4* p, f4 v) {
   u64 hi = ((u64)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
   __hip_atomic_store((u64*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __hip_atomic_store((u64*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16 bytes served by this XCD's L2 (never by the CU's vector cache): enough
+// when the writer's write-through stores went through the same L2.
+__device__ __forceinline__ f4 load_l2_scope(const f4* p) {
+  u64 lo = __hip_atomic_load((const u64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  u64 hi = __hip_atomic_load((const u64*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  f4 r = {__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
+          __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
+  return r;
 }
 __device__ __forceinline__ f4 load_device_scope(const f4* p) {
   u64 lo = __hip_atomic_load((const u64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -80,7 +95,8 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   plan.grid = (int)gridDim.x;
   const int KG = plan.KG;
   const int total = plan.NT * KG;
-  const int u0 = (int)blockIdx.x * plan.gpb;
+  const int wid = xcd_work_index((int)blockIdx.x, plan.grid);
+  const int u0 = wid * plan.gpb;
   if (u0 >= total) return;
   const int u1 = min(total, u0 + plan.gpb);
 
@@ -208,34 +224,49 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     }
 
     W4A16_STAMP(5)
-    // ---- meet the other workgroups of this tile, if any.  Partial sums
-    // travel through device-scope (write-through / always-refetched) stores
-    // and loads, so no cache write-back or invalidation is needed: a wave
-    // waits until its own stores are acknowledged, the barrier collects the
-    // four waves, and only then does thread 0 take the tile's ticket.  Whoever
-    // draws the last ticket knows every other partial has already landed.
+    // ---- meet the other workgroups of this tile, if any.  Partial sums are
+    // written with device-scope (write-through) stores, so no cache write-back
+    // is needed: a wave waits until its own stores are acknowledged, the
+    // barrier collects the four waves, and only then does thread 0 take the
+    // tile's ticket.  Whoever draws the last ticket knows every other partial
+    // has already landed in memory.  Reading them back from memory is the
+    // slowest hop, so a workgroup that runs on the XCD where the dealing puts
+    // all sharers of the tile also leaves an ordinary (write-back) copy in
+    // that XCD's L2.  A ticket carries, above bit 16, whether its workgroup
+    // was anywhere else; if nobody was, the last arrival sits behind the same
+    // L2 as every copy and reads those, otherwise it refetches the
+    // write-through copies from memory.
     const int bf = tile_first_block(plan, t);
     const int bl = tile_last_block(plan, t);
     bool writer = true;
     if (bl > bf) {
-      const size_t slot_f4 = (size_t)MB * 4 * 2 * 64;
-      f4* mine = (f4*)p.scratch + (size_t)partial_slot(plan, (int)blockIdx.x, t) * slot_f4;
+      // a slot is two copies of MB*4*2*64 f4: [0] written back lazily by this
+      // XCD's L2, [1] written through to memory
+      const size_t part_f4 = (size_t)MB * 4 * 2 * 64;
+      f4* mine = (f4*)p.scratch + (size_t)partial_slot(plan, wid, t) * (2 * part_f4);
+      const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;  // HW_REG_XCC_ID[3:0]
+      const int away = xcd_range_holds((int)blockIdx.x, (int)gridDim.x, my_xcd, bf, bl) ? 0 : 0x10000;
 #pragma unroll
       for (int i = 0; i < MB; i++)
         if (16 * i + nu < p.M) {
 #pragma unroll
-          for (int h = 0; h < 2; h++)
-            store_device_scope(&mine[((i * 4 + wave) * 2 + h) * 64 + lane], res[i][h]);
+          for (int h = 0; h < 2; h++) {
+            const int at = ((i * 4 + wave) * 2 + h) * 64 + lane;
+            if (!away) mine[at] = res[i][h];
+            store_device_scope(&mine[part_f4 + at], res[i][h]);
+          }
         }
       __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
       __syncthreads();
       if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(&p.locks[t], 1, __ATOMIC_RELAXED,
+        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride], 1 + away, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       W4A16_STAMP(6)
-      writer = (s_ticket == bl - bf);
+      writer = ((s_ticket & 0xffff) == bl - bf);
       if (writer) {
+        const bool same_l2 = (s_ticket >> 16) == 0 && away == 0;
+        W4A16_NOTE(12, same_l2 ? 1 : 2)
         // add the partials in workgroup order (deterministic), fetching them
         // eight workgroups at a time so that the loads overlap
 #pragma unroll
@@ -247,11 +278,17 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 #pragma unroll
               for (int u = 0; u < 8; u++) {
                 const int b = b0 + u;
-                if (b <= bl && b != (int)blockIdx.x) {
-                  const f4* theirs =
-                      (const f4*)p.scratch + (size_t)partial_slot(plan, b, t) * slot_f4;
-                  v[u][0] = load_device_scope(&theirs[((i * 4 + wave) * 2 + 0) * 64 + lane]);
-                  v[u][1] = load_device_scope(&theirs[((i * 4 + wave) * 2 + 1) * 64 + lane]);
+                if (b <= bl && b != wid) {
+                  const f4* theirs = (const f4*)p.scratch +
+                                     (size_t)partial_slot(plan, b, t) * (2 * part_f4) +
+                                     ((i * 4 + wave) * 2) * 64 + lane;
+                  if (same_l2) {
+                    v[u][0] = load_l2_scope(theirs);
+                    v[u][1] = load_l2_scope(theirs + 64);
+                  } else {
+                    v[u][0] = load_device_scope(theirs + part_f4);
+                    v[u][1] = load_device_scope(theirs + part_f4 + 64);
+                  }
                 } else {
                   v[u][0] = res[i][0];
                   v[u][1] = res[i][1];
@@ -270,7 +307,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           }
         }
         if (tid == 0)  // counters are handed back zeroed
-          __hip_atomic_store(&p.locks[t], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(&p.locks[t * p.lock_stride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();  // s_ticket is reused by the next tile
     }
@@ -341,7 +378,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           clear_acc();
         }
       }
-      compute(d);  // a granule past the end is all zeros and adds nothing
+#pragma unroll 1
+      for (int rep = 0; rep < W4A16_COMPUTE_REPS; rep++)
+        compute(d);  // a granule past the end is all zeros and adds nothing
       if (i == 0) { W4A16_STAMP(2) }
       ckq += 4;
       while (ckq >= KG) {
