@@ -28,9 +28,6 @@
 #ifndef W4A16_NOTE
 #define W4A16_NOTE(i, v)
 #endif
-#ifndef W4A16_COMPUTE_REPS
-#define W4A16_COMPUTE_REPS 1
-#endif
 
 namespace w4a16 {
 
@@ -366,32 +363,60 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   }
 
   W4A16_STAMP(1)
-  for (int base = 0; base < n_mine; base += DEPTH) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; d++) {
-      const int i = base + d;
-      if (i < n_mine) {
-        // entering a new tile: hand over the tiles behind me first
-        while (cur_tile < ct) {
-          finish(cur_tile);
-          ++cur_tile;
-          clear_acc();
-        }
-      }
+  if constexpr (DEPTH == 2) {
+    // At most two granules per wave and both are already requested: a rolled
+    // loop over one copy of the compute code, so that the second turn runs
+    // from the instruction cache; the second granule moves into the first's
+    // registers in between.
 #pragma unroll 1
-      for (int rep = 0; rep < W4A16_COMPUTE_REPS; rep++)
-        compute(d);  // a granule past the end is all zeros and adds nothing
+    for (int i = 0; i < n_mine; i++) {
+      while (cur_tile < ct) {
+        finish(cur_tile);
+        ++cur_tile;
+        clear_acc();
+      }
+      compute(0);
       if (i == 0) { W4A16_STAMP(2) }
       ckq += 4;
       while (ckq >= KG) {
         ckq -= KG;
         ++ct;
       }
-      issue(d, it, ikq, i + DEPTH < n_mine);
-      ikq += 4;
-      while (ikq >= KG) {
-        ikq -= KG;
-        ++it;
+#pragma unroll
+      for (int r = 0; r < 4; r++) bq[0][r] = bq[1][r];
+      sq[0] = sq[1];
+#pragma unroll
+      for (int m = 0; m < MB; m++) {
+        aq[0][m][0] = aq[1][m][0];
+        aq[0][m][1] = aq[1][m][1];
+      }
+    }
+  } else {
+    for (int base = 0; base < n_mine; base += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) {
+        const int i = base + d;
+        if (i < n_mine) {
+          // entering a new tile: hand over the tiles behind me first
+          while (cur_tile < ct) {
+            finish(cur_tile);
+            ++cur_tile;
+            clear_acc();
+          }
+        }
+        compute(d);  // a granule past the end is all zeros and adds nothing
+        if (i == 0) { W4A16_STAMP(2) }
+        ckq += 4;
+        while (ckq >= KG) {
+          ckq -= KG;
+          ++ct;
+        }
+        issue(d, it, ikq, i + DEPTH < n_mine);
+        ikq += 4;
+        while (ikq >= KG) {
+          ikq -= KG;
+          ++it;
+        }
       }
     }
   }
