@@ -71,12 +71,64 @@ __device__ __forceinline__ f4 load_device_scope(const f4* p) {
 
 }  // namespace
 
+// With one row block the activations of a granule travel through registers
+// and are transposed into LDS just before use (2 KiB per wave, inside the
+// 32 KiB that the cross-wave reduction uses later; barriers separate the two).
+// With more row blocks that would cost 8 registers per row block and ring
+// slot, so the activations are loaded straight into an LDS ring instead
+// (buffer_load ... lds, 16 bytes per lane) and never occupy a register before
+// they are an MFMA operand.
+template <int MB, int DEPTH>
+struct StreamLds {
+  static constexpr bool kDmaA = MB >= 2;
+  static constexpr int kReduceBytes = 32768;
+  static constexpr int kRingBytesPerWave = kDmaA ? DEPTH * MB * 2048 : 0;
+  static constexpr int kBytes = kReduceBytes + 4 * kRingBytesPerWave;
+};
+
+// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at
+// dst + 16*l (dst is wave-uniform).  The instruction's immediate offset is left
+// at zero: the hardware would add it to the LDS address as well.  (This and the
+// two helpers below are empty in the host pass, which only needs the kernels'
+// launch stubs.)
+__device__ __forceinline__ void ring_load(__amdgpu_buffer_rsrc_t rsrc, char* dst, int voffset,
+                                          int soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
+#endif
+}
+
+// The two halves of an MFMA activation operand from the LDS ring (dword kg of
+// chunks 0,1 and of chunks 2,3 of a row), and the wait for them.  Written as
+// assembly because the compiler must not treat them as LDS reads that depend
+// on every ring load in flight.
+__device__ __forceinline__ void ring_read(unsigned at, i2& lo, i2& hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile(
+      "ds_read2st64_b32 %0, %2 offset1:1\n\t"
+      "ds_read2st64_b32 %1, %2 offset0:2 offset1:3"
+      : "=v"(lo), "=v"(hi)
+      : "v"(at)
+      : "memory");
+#endif
+}
+// wait until at most PENDING later LDS reads are outstanding
+template <int PENDING>
+__device__ __forceinline__ void ring_read_wait(i2& lo, i2& hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(PENDING));
+#endif
+}
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
+constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
 template <int MB, bool GROUP, int DEPTH>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
-  // A staging (4 waves x MB x 2 KiB) and the cross-wave reduction (32 KiB)
-  // use the same LDS; barriers separate the two uses.
-  __shared__ __attribute__((aligned(16))) char smem[32768];
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH>::kBytes
   __shared__ int s_ticket;
+  constexpr bool kDmaA = StreamLds<MB, DEPTH>::kDmaA;
 
   W4A16_STAMP_DECL
   const int tid = threadIdx.x;
@@ -106,27 +158,40 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   // per-lane parts of the addresses; the rest is wave-uniform
   const int b_lane = 64 * nu + 16 * kg;
   const int s_lane = 16 * nu;
-  // activation staging: lane (row = lane/4, ax = lane%4) fetches 16-byte
-  // chunks ax and ax+4 of the 128-byte k run of its row
-  const int ax = lane & 3;
+  // Activation staging.  Register path: lane (row = lane/4, ax = lane%4)
+  // fetches 16-byte chunks ax and ax+4 of the 128-byte k run of its row and
+  // writes their dwords to [step][kg'][row][ax], so that MFMA lane (kg, row nu)
+  // reads its operand with one 16-byte access at a_rd.
+  // LDS-ring path: lane (kg, nu) fetches chunk kg of the 64-byte k run of row
+  // nu; the hardware puts lane l's 16 bytes at 16*l, i.e. [chunk][row].  MFMA
+  // lane (kg, nu) then needs dword kg of the four chunks of its row:
+  // 256*c + 16*nu + 4*kg, two ds_read2st64_b32 and no bank conflict.
+  const int ax = kDmaA ? kg : (lane & 3);
   int a_lane[MB];
 #pragma unroll
   for (int i = 0; i < MB; i++) {
-    int r = 16 * i + (lane >> 2);
+    int r = 16 * i + (kDmaA ? nu : (lane >> 2));
     r = r < p.M ? r : p.M - 1;  // rows past M are never written back
     a_lane[i] = r * p.K * 2 + 16 * ax;
   }
-  char* lds_a = smem + wave * (MB * 2048);
-  // write position of dword kg' of a chunk: [step][kg'][row][ax]
+  char* lds_a = kDmaA ? smem + StreamLds<MB, DEPTH>::kReduceBytes +
+                            wave * StreamLds<MB, DEPTH>::kRingBytesPerWave
+                      : smem + wave * (MB * 2048);
   const int a_wr = ((lane >> 2) * 4 + ax) * 4;
-  // read position of the operand of MFMA lane (kg, row nu)
-  const int a_rd = (kg * 16 + nu) * 16;
+  const int a_rd = kDmaA ? 16 * nu + 4 * kg : (kg * 16 + nu) * 16;
+  if constexpr (kDmaA) {
+    // A granule that does not exist multiplies zero weights with whatever its
+    // ring slot holds, so the ring must never hold NaN or Inf bit patterns.
+    for (int o = lane * 16; o < StreamLds<MB, DEPTH>::kRingBytesPerWave; o += 1024)
+      *(i4*)(lds_a + o) = (i4){0, 0, 0, 0};
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): zeros are in before the first ring load
+  }
 
   const DequantConsts dc;
 
   i4 bq[DEPTH][4];
   i4 sq[DEPTH];
-  i4 aq[DEPTH][MB][2];
+  i4 aq[kDmaA ? 1 : DEPTH][MB][2];  // unused on the LDS-ring path
 
   // request granule kq of tile t into ring slot `slot`; straight-line code, so
   // that every turn of the ring issues exactly the same loads in the same order
@@ -143,9 +208,15 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
                                                        ((kq >> 1) * p.N + kTileN * t) * 2, 0);
 #pragma unroll
     for (int i = 0; i < MB; i++) {
-      aq[slot][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq, 0);
-      aq[slot][i][1] =
-          __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq + 64, 0);
+      if constexpr (kDmaA) {
+        char* dst = lds_a + (slot * MB + i) * 2048;
+        ring_load(rA, dst, a_lane[i] | inv, 128 * kq);
+        ring_load(rA, dst + 1024, a_lane[i] | inv, 128 * kq + 64);
+      } else {
+        aq[slot][i][0] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq, 0);
+        aq[slot][i][1] =
+            __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, 128 * kq + 64, 0);
+      }
     }
     // keep the groups in issue order: the in-order load counter is only exact
     // if a slot's loads are never moved behind those of a later slot
@@ -160,21 +231,59 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       for (int j = 0; j < 8; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
   };
 
+  // loads of one ring slot: 4 weight rows, the scales, 2 per row block
+  constexpr int kLoadsPerSlot = 4 + (GROUP ? 1 : 0) + 2 * MB;
+
   auto compute = [&](int slot) {
-    // activations: registers -> LDS in MFMA k-slot order
+    // LDS-ring path: the operands of both k steps are fetched up front; the
+    // wait for the second step's comes after the first step's MFMAs
+    i2 lo[2][MB], hi[2][MB];
+    if constexpr (kDmaA) {
+      // The ring loads of this slot are DEPTH-1 slots old: everything but the
+      // loads issued since has landed.  (The compiler cannot see that LDS is
+      // written by those loads, so the wait and the LDS reads are explicit.)
+      __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm((DEPTH - 1) * kLoadsPerSlot));
 #pragma unroll
-    for (int i = 0; i < MB; i++)
+      for (int h = 0; h < 2; h++) {
 #pragma unroll
-      for (int h = 0; h < 2; h++)
+        for (int i = 0; i < MB; i++) {
+          const unsigned at =
+              (unsigned)(size_t)(lds_a + (slot * MB + i) * 2048 + h * 1024 + a_rd);
+          ring_read(at, lo[h][i], hi[h][i]);
+        }
+      }
+      // LDS reads complete in order: all but the 2*MB reads of the second step
 #pragma unroll
-        for (int g = 0; g < 4; g++)
-          *(int*)(lds_a + i * 2048 + h * 1024 + g * 256 + a_wr) = aq[slot][i][h][g];
+      for (int i = 0; i < MB; i++) ring_read_wait<2 * MB>(lo[0][i], hi[0][i]);
+    } else {
+      // activations: registers -> LDS in MFMA k-slot order
+#pragma unroll
+      for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+          for (int g = 0; g < 4; g++)
+            *(int*)(lds_a + i * 2048 + h * 1024 + g * 256 + a_wr) = aq[slot][i][h][g];
+    }
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       h8 af[MB];
+      if constexpr (kDmaA) {
+        if (h == 1) {
+          __builtin_amdgcn_sched_barrier(0);  // keep the wait behind the first step's MFMAs
 #pragma unroll
-      for (int i = 0; i < MB; i++)
-        af[i] = __builtin_bit_cast(h8, *(const i4*)(lds_a + i * 2048 + h * 1024 + a_rd));
+          for (int i = 0; i < MB; i++) ring_read_wait<0>(lo[1][i], hi[1][i]);
+        }
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+          i4 v = {lo[h][i][0], lo[h][i][1], hi[h][i][0], hi[h][i][1]};
+          af[i] = __builtin_bit_cast(h8, v);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+          af[i] = __builtin_bit_cast(h8, *(const i4*)(lds_a + i * 2048 + h * 1024 + a_rd));
+      }
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         h2 s2 = GROUP ? as_h2(sq[slot][j]) : (h2){(half_t)1.f, (half_t)1.f};
@@ -363,7 +472,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   }
 
   W4A16_STAMP(1)
-  if constexpr (DEPTH == 2) {
+  if constexpr (DEPTH == 2 && !kDmaA) {
     // At most two granules per wave and both are already requested: a rolled
     // loop over one copy of the compute code, so that the second turn runs
     // from the instruction cache; the second granule moves into the first's
@@ -428,17 +537,31 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   W4A16_STAMP(8)
 }
 
+template <int MB, bool GROUP, int DEPTH>
+static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
+  constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
+  if (lds > 65536) {
+    // more than the default limit of dynamic LDS: raised once per device
+    static bool raised[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 3;
+    if (!raised[dev]) {
+      if (hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return 3;
+      raised[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), lds, stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
 template <int MB, bool GROUP>
 static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
   // ring depth: shallow when a wave only ever sees a couple of granules
   const int per_wave = (a.gpb + 3) / 4;
-  if (per_wave <= 2) {
-    hipLaunchKernelGGL((stream_kernel<MB, GROUP, 2>), dim3(grid), dim3(256), 0, stream, a);
-  } else {
-    constexpr int DEPTH = MB <= 2 ? 4 : 3;
-    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), 0, stream, a);
-  }
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  if (per_wave <= 2) return launch_variant<MB, GROUP, 2>(a, grid, stream);
+  return launch_variant<MB, GROUP, (MB <= 2 ? 4 : 3)>(a, grid, stream);
 }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream) {
