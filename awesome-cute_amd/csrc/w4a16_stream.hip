@@ -121,6 +121,15 @@ __device__ __forceinline__ void ring_read_wait(i2& lo, i2& hi) {
 #endif
 }
 
+// Workgroup barrier for data exchanged through LDS only: waits for this wave's
+// LDS accesses, not for its global loads (__syncthreads would drain the whole
+// prefetch ring).
+__device__ __forceinline__ void lds_barrier() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#endif
+}
+
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
@@ -311,14 +320,14 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // (j = w, h = 0/1) of every row block
     f4 res[MB][2];
     W4A16_STAMP(3)
-    __syncthreads();
+    lds_barrier();
     W4A16_STAMP(4)
 #pragma unroll
     for (int i = 0; i < MB; i++) {
       f4* red = (f4*)smem;
 #pragma unroll
       for (int j = 0; j < 8; j++) red[(wave * 8 + j) * 64 + lane] = acc[i][j];
-      __syncthreads();
+      lds_barrier();
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         f4 v = red[(0 * 8 + 2 * wave + h) * 64 + lane];
@@ -326,7 +335,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         for (int w = 1; w < 4; w++) v += red[(w * 8 + 2 * wave + h) * 64 + lane];
         res[i][h] = v;
       }
-      __syncthreads();
+      lds_barrier();
     }
 
     W4A16_STAMP(5)
