@@ -72,11 +72,6 @@ float* scratch_for(int dev, hipStream_t stream) {
   return p;
 }
 
-int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v && *v ? atoi(v) : dflt;
-}
-
 // Shape checks in the order the reference performs them
 // (marlin_cute_kernel.cu:39-60, 95-107).
 int check_shape(int m, int n, int k, int groupsize, int& thread_k, int& thread_n) {
@@ -306,6 +301,10 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[4] = pl.sp.KG;
   out[5] = pl.launches;
   return rc;
+}
+
+void marlin_amd_work_order(int grid, int* out) {
+  for (int b = 0; b < grid; b++) out[b] = xcd_work_index(b, grid);
 }
 
 const char* marlin_amd_last_error(void) { return g_last_error; }

@@ -30,6 +30,8 @@ _lib.marlin_amd_check.restype = _I
 _lib.marlin_amd_check.argtypes = [_I] * 6
 _lib.marlin_amd_plan.restype = _I
 _lib.marlin_amd_plan.argtypes = [_I] * 8 + [_P]
+_lib.marlin_amd_work_order.restype = None
+_lib.marlin_amd_work_order.argtypes = [_I, _P]
 _lib.marlin_amd_last_error.restype = ctypes.c_char_p
 _lib.marlin_amd_version.restype = ctypes.c_char_p
 
@@ -191,6 +193,13 @@ def replace_linear(module, name_filter=lambda n: True, groupsize=-1, name=''):
 def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
     """Return code marlin_gemm would give for these sizes (no GPU touched)."""
     return _lib.marlin_amd_check(m, n, k, groupsize, thread_k, thread_n)
+
+
+def work_order(grid):
+    """Work index of every workgroup of a streaming launch of `grid` workgroups."""
+    out = (ctypes.c_int * grid)()
+    _lib.marlin_amd_work_order(grid, out)
+    return list(out)
 
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):

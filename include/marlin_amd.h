@@ -88,6 +88,16 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int *out);
 
+/*
+ * The streaming kernel's assignment of work to workgroups: out[b] is the work
+ * index of workgroup b of a launch of `grid` workgroups (work index w owns
+ * granules [w * granules_per_wg, (w + 1) * granules_per_wg) of the plan).  A
+ * permutation of 0..grid-1 in which the workgroups that the hardware deals to
+ * one XCD (b mod 8) hold consecutive indices.  No reference counterpart; for
+ * tests and tools.
+ */
+void marlin_amd_work_order(int grid, int *out);
+
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *marlin_amd_last_error(void);
 

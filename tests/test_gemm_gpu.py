@@ -149,6 +149,60 @@ def test_deterministic(env):
     assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
 
 
+def test_partition_does_not_change_the_bits(env):
+    """Partial sums are added in workgroup order by whoever arrives last, so a
+    given partition always gives the same bits; different partitions differ
+    only by fp32 reassociation (inside the tolerance)."""
+    A, q, s, B, sp = O.make_problem(16, 1024, 2048, 128, seed=21)
+    for sms in (24, 40, 256):
+        runs = [gpu_gemm(env, A, B, sp, 1024, sms=sms) for _ in range(3)]
+        assert all(np.array_equal(runs[0].view(np.uint16), r.view(np.uint16)) for r in runs[1:])
+
+
+@pytest.mark.parametrize("max_par", [1, 2, 5, 8, 16, 64])
+def test_workspace_stride_follows_max_par(env, max_par):
+    """The tile counters sit max_par ints apart (capped at 16) inside the
+    n/128*max_par ints the reference asks for (marlin_gemm.cpp:29-31): the
+    smallest legal workspace works and comes back zeroed."""
+    check(env, 16, 1024, 2048, 128, seed=max_par, max_par=max_par, sms=40)
+    check(env, 33, 512, 1024, -1, seed=max_par + 1, max_par=max_par, sms=24)
+
+
+def test_back_to_back_launches_share_scratch(env):
+    """Launches on one stream reuse the partial-sum slots (and the copies of
+    them that an XCD's L2 keeps): different inputs of one shape, and then
+    another shape, must not see each other's partial sums."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    probs = [O.make_problem(m, n, k, 128, seed) for (m, n, k, seed) in
+             [(4, 4096, 4096, 31), (4, 4096, 4096, 32), (4, 4096, 4096, 33), (40, 1024, 4096, 34),
+              (4, 4096, 4096, 35)]]
+    outs = []
+    for A, q, s, B, sp in probs:
+        n = B.shape[1] // 2
+        dC = torch.zeros((A.shape[0], n), dtype=torch.half, device=dev)
+        ws = torch.zeros(n // 128 * 16, dtype=torch.int, device=dev)
+        marlin.mul(torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev), dC,
+                   torch.from_numpy(sp).to(dev), ws)
+        outs.append((dC, ws))  # no synchronisation between the launches
+    torch.cuda.synchronize()
+    for (A, q, s, B, sp), (dC, ws) in zip(probs, outs):
+        n = B.shape[1] // 2
+        r = O.compare(dC.cpu().numpy(), O.gemm(A, B, sp, n, 128))
+        assert r.max_abs_err <= TOL * r.max_abs_ref
+        assert not ws.any().item()
+
+
+@pytest.mark.parametrize("m", [17, 31, 32, 33, 47, 48, 49, 63, 64])
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_lds_ring_row_counts(env, m, groupsize):
+    """2-4 row blocks take their activations through the LDS ring; ragged row
+    counts, a deep k (many ring turns) and a shallow one (ring never full; one
+    scale row would mean per-channel scales, so two groups at least)."""
+    check(env, m, 512, 4096, groupsize, seed=m)
+    check(env, m, 256, 256, groupsize, seed=m + 100)
+
+
 def test_config2_decode(env):
     check(env, 1, 4096, 4096, 128, seed=2)
 

@@ -32,7 +32,8 @@ def test_library_exports_every_declared_symbol(marlin):
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     names = re.findall(r"\b(marlin_\w+)\s*\(", header)
     assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
-            "marlin_amd_plan", "marlin_amd_last_error", "marlin_amd_version"} <= set(names)
+            "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_last_error",
+            "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
     for n in set(names):
         assert hasattr(lib, n), n
@@ -136,6 +137,20 @@ def test_stream_partition_properties(marlin, n, k, sms):
         tiles = np.unique(np.nonzero(owner == b)[0])
         for t in tiles[1:-1]:
             assert (owner[t] == b).all()
+
+
+@pytest.mark.parametrize("grid", [1, 2, 7, 8, 9, 15, 16, 100, 172, 224, 251, 256, 1000, 1024])
+def test_work_order_is_an_xcd_blocked_permutation(marlin, grid):
+    """Workgroup b runs on XCD b % 8; the work indices of one XCD's workgroups
+    form one run of consecutive numbers, so that the consecutive work indices
+    that share a column tile meet behind one L2."""
+    order = marlin.work_order(grid)
+    assert sorted(order) == list(range(grid))
+    start = 0
+    for x in range(8):
+        mine = [order[b] for b in range(x, grid, 8)]
+        assert mine == list(range(start, start + len(mine)))
+        start += len(mine)
 
 
 def test_plan_picks_kernels(marlin):
