@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -112,9 +113,31 @@ struct Plan {
 
 constexpr int kStreamMaxRows = 64;
 
+// 0 = choose by cost, 1 = streaming kernel (in chunks of 64 rows), 2 = prefill
+// kernel; set by marlin_amd_force_kernel (tests and tools)
+std::atomic<int> g_force_kernel{0};
+
+// Above 64 rows either kernel can do the job: the prefill kernel once, with
+// ceil(m/128) * n/256 workgroups, or the streaming kernel once per 64 rows,
+// reading the weights again every time.  Costs in us from measurements at
+// n = k = 4096: a full prefill tile column (k = 4096) takes 62 us however few
+// workgroups there are, a 64-row streaming pass 5 us + its weight bytes at
+// 2.5 TB/s.
+bool prefer_prefill(int m, int n, int k, int cus) {
+  const double rounds = ceil_div(ceil_div(m, 128) * (n / 256), cus);
+  const double t_prefill = rounds * 62.0 * k / 4096.0;
+  const double t_stream = ceil_div(m, kStreamMaxRows) * (5.0 + 0.5 * n * k / 2.5e6);
+  return t_prefill <= t_stream;
+}
+
 Plan make_plan(int m, int n, int k, int sms, int cus) {
   Plan pl;
-  if (m > kStreamMaxRows) {
+  const int force = g_force_kernel.load(std::memory_order_relaxed);
+  // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
+  // whenever m > 16, by the shape contract)
+  const bool prefill = n % 256 == 0 && (force == 2 || (force == 0 && m > kStreamMaxRows &&
+                                                       prefer_prefill(m, n, k, cus)));
+  if (prefill) {
     // MFMA-bound: one workgroup per 128 x 256 tile of C
     pl.kernel = 2;
     pl.grid = ceil_div(m, 128) * (n / 256);
@@ -301,6 +324,10 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[4] = pl.sp.KG;
   out[5] = pl.launches;
   return rc;
+}
+
+void marlin_amd_force_kernel(int which) {
+  g_force_kernel.store(which == 1 || which == 2 ? which : 0, std::memory_order_relaxed);
 }
 
 void marlin_amd_work_order(int grid, int* out) {

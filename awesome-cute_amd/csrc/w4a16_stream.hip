@@ -42,31 +42,25 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsig
 // s_waitcnt vmcnt(0) with the other counters left alone (gfx9 encoding)
 constexpr int kWaitVm0 = 0x0F70;
 
-typedef unsigned long long u64;
+// Cache policy bits of the buffer instructions on gfx950: sc0 = bit 0,
+// sc1 = bit 4.  A store with sc1 is written through to the memory that all
+// XCDs share (device scope) and a load with sc1 never returns a line held by
+// this XCD's L2; a load with sc0 alone bypasses the CU's vector cache and is
+// served by this XCD's L2.
+constexpr int kAuxL2 = 1;
+constexpr int kAuxDevice = 16;
 
-// 16 bytes as two 64-bit device-scope accesses: stores are written through to
-// memory shared by all XCDs, loads never return a line cached by this XCD's L2.
-__device__ __forceinline__ void store_device_scope(f4* p, f4 v) {
-  u64 lo = ((u64)__float_as_uint(v[1]) << 32) | __float_as_uint(v[0]);
-  u64 hi = ((u64)__float_as_uint(v[3]) << 32) | __float_as_uint(v[2]);
-  __hip_atomic_store((u64*)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store((u64*)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane of a partial-sum slot, as whole-line buffer accesses
+template <int AUX>
+__device__ __forceinline__ void store_partial(__amdgpu_buffer_rsrc_t r, int voffset, int soffset,
+                                              f4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, v), r, voffset, soffset, AUX);
 }
-// 16 bytes served by this XCD's L2 (never by the CU's vector cache): enough
-// when the writer's write-through stores went through the same L2.
-__device__ __forceinline__ f4 load_l2_scope(const f4* p) {
-  u64 lo = __hip_atomic_load((const u64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  u64 hi = __hip_atomic_load((const u64*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  f4 r = {__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
-          __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
-  return r;
-}
-__device__ __forceinline__ f4 load_device_scope(const f4* p) {
-  u64 lo = __hip_atomic_load((const u64*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  u64 hi = __hip_atomic_load((const u64*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  f4 r = {__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
-          __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
-  return r;
+template <int AUX>
+__device__ __forceinline__ f4 load_partial(__amdgpu_buffer_rsrc_t r, int voffset, int soffset) {
+  return __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(r, voffset, soffset, AUX));
 }
 
 }  // namespace
@@ -357,8 +351,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     if (bl > bf) {
       // a slot is two copies of MB*4*2*64 f4: [0] written back lazily by this
       // XCD's L2, [1] written through to memory
-      const size_t part_f4 = (size_t)MB * 4 * 2 * 64;
-      f4* mine = (f4*)p.scratch + (size_t)partial_slot(plan, wid, t) * (2 * part_f4);
+      constexpr int part_bytes = MB * 4 * 2 * 64 * 16;
+      const __amdgpu_buffer_rsrc_t rP = make_rsrc(p.scratch, 0x7fffffffu);
+      const int mine = partial_slot(plan, wid, t) * (2 * part_bytes);
       const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;  // HW_REG_XCC_ID[3:0]
       const int away = xcd_range_holds((int)blockIdx.x, (int)gridDim.x, my_xcd, bf, bl) ? 0 : 0x10000;
 #pragma unroll
@@ -366,9 +361,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         if (16 * i + nu < p.M) {
 #pragma unroll
           for (int h = 0; h < 2; h++) {
-            const int at = ((i * 4 + wave) * 2 + h) * 64 + lane;
-            if (!away) mine[at] = res[i][h];
-            store_device_scope(&mine[part_f4 + at], res[i][h]);
+            const int at = (((i * 4 + wave) * 2 + h) * 64 + lane) * 16;
+            if (!away) store_partial<0>(rP, at, mine, res[i][h]);
+            store_partial<kAuxDevice>(rP, at, mine + part_bytes, res[i][h]);
           }
         }
       __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
@@ -394,15 +389,14 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
               for (int u = 0; u < 8; u++) {
                 const int b = b0 + u;
                 if (b <= bl && b != wid) {
-                  const f4* theirs = (const f4*)p.scratch +
-                                     (size_t)partial_slot(plan, b, t) * (2 * part_f4) +
-                                     ((i * 4 + wave) * 2) * 64 + lane;
+                  const int theirs = partial_slot(plan, b, t) * (2 * part_bytes);
+                  const int at = (((i * 4 + wave) * 2) * 64 + lane) * 16;
                   if (same_l2) {
-                    v[u][0] = load_l2_scope(theirs);
-                    v[u][1] = load_l2_scope(theirs + 64);
+                    v[u][0] = load_partial<kAuxL2>(rP, at, theirs);
+                    v[u][1] = load_partial<kAuxL2>(rP, at + 1024, theirs);
                   } else {
-                    v[u][0] = load_device_scope(theirs + part_f4);
-                    v[u][1] = load_device_scope(theirs + part_f4 + 64);
+                    v[u][0] = load_partial<kAuxDevice>(rP, at, theirs + part_bytes);
+                    v[u][1] = load_partial<kAuxDevice>(rP, at + 1024, theirs + part_bytes);
                   }
                 } else {
                   v[u][0] = res[i][0];

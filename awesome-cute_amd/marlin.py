@@ -30,6 +30,8 @@ _lib.marlin_amd_check.restype = _I
 _lib.marlin_amd_check.argtypes = [_I] * 6
 _lib.marlin_amd_plan.restype = _I
 _lib.marlin_amd_plan.argtypes = [_I] * 8 + [_P]
+_lib.marlin_amd_force_kernel.restype = None
+_lib.marlin_amd_force_kernel.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
 _lib.marlin_amd_work_order.argtypes = [_I, _P]
 _lib.marlin_amd_last_error.restype = ctypes.c_char_p
@@ -193,6 +195,11 @@ def replace_linear(module, name_filter=lambda n: True, groupsize=-1, name=''):
 def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
     """Return code marlin_gemm would give for these sizes (no GPU touched)."""
     return _lib.marlin_amd_check(m, n, k, groupsize, thread_k, thread_n)
+
+
+def force_kernel(which):
+    """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel (process-wide)."""
+    _lib.marlin_amd_force_kernel(int(which))
 
 
 def work_order(grid):

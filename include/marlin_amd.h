@@ -98,6 +98,14 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
  */
 void marlin_amd_work_order(int grid, int *out);
 
+/*
+ * Which kernel marlin_gemm uses, process-wide: 0 = choose by cost (default),
+ * 1 = the streaming kernel, 64 rows per launch, 2 = the prefill kernel (needs
+ * prob_n % 256 == 0, else the streaming kernel is used).  No reference
+ * counterpart; for tests and tools.
+ */
+void marlin_amd_force_kernel(int which);
+
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *marlin_amd_last_error(void);
 
