@@ -119,14 +119,21 @@ std::atomic<int> g_force_kernel{0};
 
 // Above 64 rows either kernel can do the job: the prefill kernel once, with
 // ceil(m/128) * n/256 workgroups, or the streaming kernel once per 64 rows,
-// reading the weights again every time.  Costs in us from measurements at
-// n = k = 4096: a full prefill tile column (k = 4096) takes 62 us however few
-// workgroups there are, a 64-row streaming pass 5 us + its weight bytes at
-// 2.5 TB/s.
+// reading the weights again every time.  Costs in us fitted to measurements
+// (n, k in {4096, 11008}, m = 64 ... 1024): a round of prefill workgroups
+// takes 6 + 0.0108 k whatever their number up to the CU count; a 64-row
+// streaming pass 11.6 + 0.52 per MB of packed weights, a last pass of at most
+// 16 rows 5 + 0.25 per MB.
 bool prefer_prefill(int m, int n, int k, int cus) {
   const double rounds = ceil_div(ceil_div(m, 128) * (n / 256), cus);
-  const double t_prefill = rounds * 62.0 * k / 4096.0;
-  const double t_stream = ceil_div(m, kStreamMaxRows) * (5.0 + 0.5 * n * k / 2.5e6);
+  const double t_prefill = rounds * (6.0 + 0.0108 * k);
+  const double mb_weights = 0.5e-6 * n * k;
+  const int tail = m % kStreamMaxRows;
+  double t_stream = (m / kStreamMaxRows) * (11.6 + 0.52 * mb_weights);
+  if (tail > 16)
+    t_stream += 11.6 + 0.52 * mb_weights;
+  else if (tail > 0)
+    t_stream += 5.0 + 0.25 * mb_weights;
   return t_prefill <= t_stream;
 }
 

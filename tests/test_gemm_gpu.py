@@ -203,6 +203,22 @@ def test_lds_ring_row_counts(env, m, groupsize):
     check(env, m, 256, 256, groupsize, seed=m + 100)
 
 
+@pytest.mark.parametrize("which", [1, 2])
+@pytest.mark.parametrize("m", [65, 100, 128, 200, 257])
+def test_either_kernel_above_64_rows(env, which, m):
+    """Above 64 rows the host picks the streaming kernel (64 rows per launch,
+    the reference's own scheme, marlin_cute_kernel.cu:70-93) or the prefill
+    kernel by cost; both must give the reference's result for any row count."""
+    torch, marlin = env
+    marlin.force_kernel(which)
+    try:
+        assert marlin.plan(m, 512, 1024, 128)[1]["kernel"] == which
+        check(env, m, 512, 1024, 128, seed=m + which)
+        check(env, m, 256, 768, -1, seed=m + which + 7)
+    finally:
+        marlin.force_kernel(0)
+
+
 def test_config2_decode(env):
     check(env, 1, 4096, 4096, 128, seed=2)
 

@@ -32,7 +32,8 @@ def test_library_exports_every_declared_symbol(marlin):
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     names = re.findall(r"\b(marlin_\w+)\s*\(", header)
     assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
-            "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_last_error",
+            "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_force_kernel",
+            "marlin_amd_last_error",
             "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
     for n in set(names):
@@ -151,6 +152,24 @@ def test_work_order_is_an_xcd_blocked_permutation(marlin, grid):
         mine = [order[b] for b in range(x, grid, 8)]
         assert mine == list(range(start, start + len(mine)))
         start += len(mine)
+
+
+def test_kernel_choice_above_64_rows(marlin):
+    """Few rows over wide weights go through the streaming kernel in 64-row
+    launches, many rows through the prefill kernel; the force knob overrides."""
+    assert marlin.plan(128, 4096, 4096, 128)[1] == {
+        **marlin.plan(64, 4096, 4096, 128)[1], "launches": 2}
+    assert marlin.plan(1024, 4096, 4096, 128)[1]["kernel"] == 2
+    try:
+        marlin.force_kernel(1)
+        rc, p = marlin.plan(2048, 4096, 4096, 128)
+        assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32
+        marlin.force_kernel(2)
+        rc, p = marlin.plan(100, 512, 1024, 128)
+        assert rc == 0 and p["kernel"] == 2 and p["grid"] == 2
+        assert marlin.plan(16, 128, 512, 128)[1]["kernel"] == 1  # n = 128: no 256-wide tile
+    finally:
+        marlin.force_kernel(0)
 
 
 def test_plan_picks_kernels(marlin):
