@@ -12,7 +12,8 @@ the eager (one host call per step) rate is reported next to it.
 Prints ONE JSON line: the headline workload is BASELINE config 2 (decode,
 M=1, N=K=4096, group 128), with `roofline` for its kernel and `cpu_baseline`
 from the CPU oracle; `shapes` carries the other points of the metric
-(M=16 and M=2048 at N=K=4096) measured the same way.
+(M=16 and M=2048 at N=K=4096) and BASELINE configs 3 and 5, measured the same
+way.
 """
 import argparse
 import json
@@ -173,7 +174,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--shape", default="headline",
-                    help="headline (decode + batch16 + prefill) or one of: " + ", ".join(SHAPES))
+                    help="headline (decode, then the other BASELINE shapes) or one of: " +
+                         ", ".join(SHAPES))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the "
@@ -190,7 +192,7 @@ def main():
         sys.exit("bench.py: no GPU visible")
 
     if args.shape == "headline":
-        main_name, others = "decode", ["batch16", "prefill"]
+        main_name, others = "decode", ["batch16", "prefill", "mlp_up", "mlp_down", "large_g128"]
     else:
         main_name, others = args.shape, []
 
