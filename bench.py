@@ -110,20 +110,26 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True):
         eager_ms = (time.perf_counter() - t0) * 1e3 / steps
         eager_dev_ms = e0.elapsed_time(e1) / steps
 
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph, stream=side):
-        for i in range(steps):
-            call(i)
-    for _ in range(2):
+    def graph_ms(fn):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(steps):
+                fn(i)
+        for _ in range(2):
+            graph.replay()
+        torch.cuda.synchronize()
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        cur = torch.cuda.current_stream()
+        g0.record(cur)
         graph.replay()
-    torch.cuda.synchronize()
-    g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    cur = torch.cuda.current_stream()
-    g0.record(cur)
-    graph.replay()
-    g1.record(cur)
-    torch.cuda.synchronize()
-    ms = g0.elapsed_time(g1) / steps
+        g1.record(cur)
+        torch.cuda.synchronize()
+        return g0.elapsed_time(g1) / steps
+
+    ms = graph_ms(call)
+    # the same launches over one weight buffer, which then stays in the 256 MB
+    # Infinity Cache / L2: the figure kernel timings on other hardware usually are
+    resident_ms = graph_ms(lambda i: call(0)) if bound == "hbm" and nbuf > 1 else None
 
     flops = 2.0 * M * N * K
     res = {
@@ -133,6 +139,7 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True):
         "weight_GBps": weight_bytes / (ms * 1e-3) / 1e9,
         "tflops": flops / (ms * 1e-3) / 1e12,
         "weight_buffers_rotated": nbuf,
+        "cache_resident_us_per_launch": None if resident_ms is None else resident_ms * 1e3,
     }
     if bound == "hbm":
         ach = res["weight_GBps"]
@@ -211,6 +218,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    prop = torch.cuda.get_device_properties(0)
+    # cross-check of the published matrix peak: CUs x 4 SIMDs x 1024 fp16 flop per clock x clock
+    clock_khz = getattr(prop, "clock_rate", None)  # not exposed by every torch build
+    peaks = {"hbm_GBps": HBM_PEAK_GBPS, "mfma_fp16_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
+             "device": prop.name, "compute_units": prop.multi_processor_count,
+             "clock_MHz": None if clock_khz is None else clock_khz / 1e3,
+             "mfma_fp16_TFLOPs_at_2400MHz": prop.multi_processor_count * 4 * 1024 * 2.4e9 / 1e12,
+             "mfma_fp16_TFLOPs_from_clock": None if clock_khz is None else
+                 prop.multi_processor_count * 4 * 1024 * clock_khz * 1e3 / 1e12}
     head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup)
     shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup) for n in others]
 
@@ -227,6 +243,8 @@ def main():
                    "weight_buffers_rotated": head["weight_buffers_rotated"],
                    "timing": "K launches in one HIP graph, HIP events on the launch stream"},
         "tflops": head["tflops"], "weight_GBps": head["weight_GBps"],
+        "cache_resident_us_per_launch": head["cache_resident_us_per_launch"],
+        "peaks": peaks,
         "eager_ms_per_step": head["eager_ms_per_step"],
         "roofline": head["roofline"],
         "shapes": shapes,
