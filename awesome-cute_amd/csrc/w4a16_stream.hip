@@ -377,43 +377,50 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       if (writer) {
         const bool same_l2 = (s_ticket >> 16) == 0 && away == 0;
         W4A16_NOTE(12, same_l2 ? 1 : 2)
-        // add the partials in workgroup order (deterministic), fetching them
-        // eight workgroups at a time so that the loads overlap
+        // Add the partials in workgroup order (deterministic).  They are fetched
+        // eight workgroups at a time, and the next row block's are requested
+        // before this row block's are added, so that the loads overlap.  Rows
+        // past M are requested out of range (zeros, no traffic).
+        f4 sum[MB][2];
+        for (int b0 = bf; b0 <= bl; b0 += 8) {
+          f4 v[2][8][2];
+          auto fetch = [&](int i, f4 (&dst)[8][2]) {
+            const int at = ((((i * 4 + wave) * 2) * 64 + lane) * 16) | (16 * i + nu < p.M ? 0 : kOob);
 #pragma unroll
-        for (int i = 0; i < MB; i++) {
-          if (16 * i + nu < p.M) {
-            f4 sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-            for (int b0 = bf; b0 <= bl; b0 += 8) {
-              f4 v[8][2];
-#pragma unroll
-              for (int u = 0; u < 8; u++) {
-                const int b = b0 + u;
-                if (b <= bl && b != wid) {
-                  const int theirs = partial_slot(plan, b, t) * (2 * part_bytes);
-                  const int at = (((i * 4 + wave) * 2) * 64 + lane) * 16;
-                  if (same_l2) {
-                    v[u][0] = load_partial<kAuxL2>(rP, at, theirs);
-                    v[u][1] = load_partial<kAuxL2>(rP, at + 1024, theirs);
-                  } else {
-                    v[u][0] = load_partial<kAuxDevice>(rP, at, theirs + part_bytes);
-                    v[u][1] = load_partial<kAuxDevice>(rP, at + 1024, theirs + part_bytes);
-                  }
+            for (int u = 0; u < 8; u++) {
+              const int b = b0 + u;
+              if (b <= bl && b != wid) {
+                const int theirs = partial_slot(plan, b, t) * (2 * part_bytes);
+                if (same_l2) {
+                  dst[u][0] = load_partial<kAuxL2>(rP, at, theirs);
+                  dst[u][1] = load_partial<kAuxL2>(rP, at + 1024, theirs);
                 } else {
-                  v[u][0] = res[i][0];
-                  v[u][1] = res[i][1];
+                  dst[u][0] = load_partial<kAuxDevice>(rP, at, theirs + part_bytes);
+                  dst[u][1] = load_partial<kAuxDevice>(rP, at + 1024, theirs + part_bytes);
                 }
-              }
-#pragma unroll
-              for (int u = 0; u < 8; u++) {
-                if (b0 + u <= bl) {
-                  sum[0] = (b0 + u == bf) ? v[u][0] : sum[0] + v[u][0];
-                  sum[1] = (b0 + u == bf) ? v[u][1] : sum[1] + v[u][1];
-                }
+              } else {
+                dst[u][0] = res[i][0];
+                dst[u][1] = res[i][1];
               }
             }
-            res[i][0] = sum[0];
-            res[i][1] = sum[1];
+          };
+          fetch(0, v[0]);
+#pragma unroll
+          for (int i = 0; i < MB; i++) {
+            if (i + 1 < MB) fetch(i + 1, v[(i + 1) & 1]);
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+              if (b0 + u <= bl) {
+                sum[i][0] = (b0 + u == bf) ? v[i & 1][u][0] : sum[i][0] + v[i & 1][u][0];
+                sum[i][1] = (b0 + u == bf) ? v[i & 1][u][1] : sum[i][1] + v[i & 1][u][1];
+              }
+            }
           }
+        }
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+          res[i][0] = sum[i][0];
+          res[i][1] = sum[i][1];
         }
         if (tid == 0)  // counters are handed back zeroed
           __hip_atomic_store(&p.locks[t * p.lock_stride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
