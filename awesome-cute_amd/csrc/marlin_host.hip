@@ -38,12 +38,25 @@ struct Scratch {
 };
 struct DeviceState {
   int cus = 0;
+  bool configured = false;  // kernels' LDS limits raised on this device
   std::vector<Scratch> scratch;
 };
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 
 constexpr size_t kScratchBytes = (size_t)2 * kMaxStreamGrid * stream_slot_bytes(4);
+
+// With `dev` current: raise the dynamic-LDS limit of the kernels that need it.
+bool configure_device(int dev) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_dev[dev].configured) return true;
+  if (configure_stream_kernels() != 0 || configure_prefill_kernels() != 0) {
+    set_error(hipGetLastError(), "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    return false;
+  }
+  g_dev[dev].configured = true;
+  return true;
+}
 
 int device_cus(int dev) {
   std::lock_guard<std::mutex> lk(g_mu);
@@ -217,7 +230,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   }
   int cus = device_cus(dev);
   rc = MARLIN_ERR_RUNTIME;
-  if (cus > 0) {
+  if (cus > 0 && configure_device(dev)) {
     Plan pl = make_plan(m, n, k, sms, cus);
     float* scratch = pl.kernel == 1 ? scratch_for(dev, stream) : nullptr;
     if (pl.kernel == 2) {

@@ -173,6 +173,11 @@ struct GemmArgs {
 constexpr size_t stream_partial_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
 constexpr size_t stream_slot_bytes(int mb) { return 2 * stream_partial_bytes(mb); }
 
+// Per-device set-up of the kernels that need more dynamic LDS than the default
+// limit; call once with the device current before the first launch on it.
+int configure_stream_kernels();
+int configure_prefill_kernels();
+
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream);
 

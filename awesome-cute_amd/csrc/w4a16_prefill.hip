@@ -341,20 +341,20 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   W4A16_PF_TEXIT
 }
 
+int configure_prefill_kernels() {
+  // more LDS than the default per-workgroup limit: opt in per kernel and device
+  if (hipFuncSetAttribute((const void*)prefill_kernel<true>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess ||
+      hipFuncSetAttribute((const void*)prefill_kernel<false>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess)
+    return 3;
+  return 0;
+}
+
 int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream) {
   const int tiles_m = ceil_div(a.M, kPfTileM);
   const int tiles_n = a.N / kPfTileN;
   const int grid = tiles_m * tiles_n;
-  // more LDS than the default per-workgroup limit: opt in once per kernel
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute((const void*)prefill_kernel<true>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)prefill_kernel<false>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess)
-      return 3;
-    configured = true;
-  }
   if (group)
     hipLaunchKernelGGL(prefill_kernel<true>, dim3(grid), dim3(512), kPfLdsBytes, stream, a,
                        tiles_m, tiles_n);

@@ -550,20 +550,37 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 template <int MB, bool GROUP, int DEPTH>
 static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
   constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
-  if (lds > 65536) {
-    // more than the default limit of dynamic LDS: raised once per device
-    static bool raised[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 3;
-    if (!raised[dev]) {
-      if (hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-        return 3;
-      raised[dev] = true;
-    }
-  }
   hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), lds, stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+// ring depth of the deep variant of each row-block count
+template <int MB>
+constexpr int deep_ring() {
+  return MB <= 2 ? 4 : 3;
+}
+
+template <int MB, bool GROUP, int DEPTH>
+static int configure_variant() {
+  constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
+  if (lds <= 65536) return 0;  // within the default limit of dynamic LDS
+  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH>,
+                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess
+             ? 0
+             : 3;
+}
+template <int MB>
+static int configure_row_blocks() {
+  return configure_variant<MB, false, 2>() | configure_variant<MB, true, 2>() |
+         configure_variant<MB, false, deep_ring<MB>()>() |
+         configure_variant<MB, true, deep_ring<MB>()>();
+}
+
+int configure_stream_kernels() {
+  return (configure_row_blocks<1>() | configure_row_blocks<2>() | configure_row_blocks<3>() |
+          configure_row_blocks<4>())
+             ? 3
+             : 0;
 }
 
 template <int MB, bool GROUP>
@@ -571,7 +588,7 @@ static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
   // ring depth: shallow when a wave only ever sees a couple of granules
   const int per_wave = (a.gpb + 3) / 4;
   if (per_wave <= 2) return launch_variant<MB, GROUP, 2>(a, grid, stream);
-  return launch_variant<MB, GROUP, (MB <= 2 ? 4 : 3)>(a, grid, stream);
+  return launch_variant<MB, GROUP, deep_ring<MB>()>(a, grid, stream);
 }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream) {
