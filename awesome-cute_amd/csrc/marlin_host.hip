@@ -44,7 +44,12 @@ struct DeviceState {
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 
-constexpr size_t kScratchBytes = (size_t)2 * kMaxStreamGrid * stream_slot_bytes(4);
+constexpr size_t kPartialBytes = (size_t)2 * kMaxStreamGrid * stream_slot_bytes(4);
+// behind the partial sums: the tile counters of the prefill kernel's k slices
+// (the caller's workspace has one counter per 128 columns, too few for tiles
+// of many rows), zero whenever no launch is in flight
+constexpr int kMaxPrefillTiles = 16384;
+constexpr size_t kScratchBytes = kPartialBytes + (size_t)kMaxPrefillTiles * sizeof(int);
 
 // With `dev` current: raise the dynamic-LDS limit of the kernels that need it.
 bool configure_device(int dev) {
@@ -80,6 +85,12 @@ float* scratch_for(int dev, hipStream_t stream) {
   hipError_t e = hipMalloc((void**)&p, kScratchBytes);
   if (e != hipSuccess) {
     set_error(e, "hipMalloc(scratch)");
+    return nullptr;
+  }
+  e = hipMemset((char*)p + kPartialBytes, 0, kScratchBytes - kPartialBytes);
+  if (e != hipSuccess) {
+    set_error(e, "hipMemset(scratch)");
+    (void)hipFree(p);
     return nullptr;
   }
   g_dev[dev].scratch.push_back({stream, p});
@@ -122,6 +133,8 @@ struct Plan {
   int grid;
   StreamPlan sp;
   int launches;
+  int ksplit;     // prefill: slices of the k range per tile
+  int tile_rows;  // prefill: rows of C per workgroup
 };
 
 constexpr int kStreamMaxRows = 64;
@@ -150,6 +163,22 @@ bool prefer_prefill(int m, int n, int k, int cus) {
   return t_prefill <= t_stream;
 }
 
+// Slices of the k range per prefill tile.  A slice must be at least 256 deep
+// (two 64-deep stages for each half of the workgroup) and the tile counters
+// and partial-sum slots must fit; within that, 0 = by cost.
+std::atomic<int> g_force_k_slices{0};
+
+int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
+  int most = k / 256;
+  if (most > 8) most = 8;
+  while (most > 1 && (size_t)tiles * most * tile_rows * 256 * 4 > kPartialBytes) --most;
+  if (most < 1 || tiles > kMaxPrefillTiles) return 1;
+  const int force = g_force_k_slices.load(std::memory_order_relaxed);
+  if (force > 0) return force < most ? force : most;
+  (void)cus;
+  return 1;
+}
+
 Plan make_plan(int m, int n, int k, int sms, int cus) {
   Plan pl;
   const int force = g_force_kernel.load(std::memory_order_relaxed);
@@ -157,10 +186,15 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   // whenever m > 16, by the shape contract)
   const bool prefill = n % 256 == 0 && (force == 2 || (force == 0 && m > kStreamMaxRows &&
                                                        prefer_prefill(m, n, k, cus)));
+  pl.ksplit = 1;
+  pl.tile_rows = 0;
   if (prefill) {
-    // MFMA-bound: one workgroup per 128 x 256 tile of C
+    // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
-    pl.grid = ceil_div(m, 128) * (n / 256);
+    pl.tile_rows = prefill_tile_rows(m);
+    const int tiles = ceil_div(m, pl.tile_rows) * (n / 256);
+    pl.ksplit = prefill_k_slices(tiles, pl.tile_rows, k, cus);
+    pl.grid = tiles * pl.ksplit;
     pl.sp = make_stream_plan(n, k, 1);
     pl.launches = 1;
     return pl;
@@ -232,8 +266,9 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0 && configure_device(dev)) {
     Plan pl = make_plan(m, n, k, sms, cus);
-    float* scratch = pl.kernel == 1 ? scratch_for(dev, stream) : nullptr;
-    if (pl.kernel == 2) {
+    float* scratch =
+        pl.kernel == 1 || pl.ksplit > 1 ? scratch_for(dev, stream) : nullptr;
+    if (pl.kernel == 2 && (pl.ksplit == 1 || scratch)) {
       GemmArgs a;
       a.A = A;
       a.B = B;
@@ -242,13 +277,13 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
       a.M = m;
       a.N = n;
       a.K = k;
-      a.locks = (int*)workspace;
-      a.lock_stride = lock_stride;
-      a.scratch = nullptr;
+      a.locks = scratch ? (int*)((char*)scratch + kPartialBytes) : nullptr;
+      a.lock_stride = 1;
+      a.scratch = scratch;
       a.gpb = 0;
-      rc = launch_prefill(a, groupsize != -1, stream);
+      rc = launch_prefill(a, groupsize != -1, pl.ksplit, stream);
       if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
-    } else if (scratch) {
+    } else if (pl.kernel == 1 && scratch) {
       rc = MARLIN_OK;
       for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
         GemmArgs a;
@@ -333,7 +368,7 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int* out) {
-  for (int i = 0; i < 6; i++) out[i] = 0;
+  for (int i = 0; i < 8; i++) out[i] = 0;
   int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
   Plan pl = make_plan(prob_m, prob_n, prob_k, sms, cus);
@@ -343,11 +378,17 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[3] = pl.sp.NT;
   out[4] = pl.sp.KG;
   out[5] = pl.launches;
+  out[6] = pl.ksplit;
+  out[7] = pl.tile_rows;
   return rc;
 }
 
 void marlin_amd_force_kernel(int which) {
   g_force_kernel.store(which == 1 || which == 2 ? which : 0, std::memory_order_relaxed);
+}
+
+void marlin_amd_force_k_slices(int slices) {
+  g_force_k_slices.store(slices > 0 ? slices : 0, std::memory_order_relaxed);
 }
 
 void marlin_amd_work_order(int grid, int* out) {

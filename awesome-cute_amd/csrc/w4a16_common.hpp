@@ -27,6 +27,7 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
 typedef int i2 __attribute__((ext_vector_type(2)));
 typedef int i4 __attribute__((ext_vector_type(4)));
 
@@ -179,6 +180,10 @@ int configure_stream_kernels();
 int configure_prefill_kernels();
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
-int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream);
+// ksplit >= 1 slices of the k range per tile; above 1 the launch needs
+// a.scratch (ksplit * tiles * tile bytes of fp32) and a.locks (one zeroed
+// counter per tile, zero again afterwards)
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
+int prefill_tile_rows(int m);  // rows of C per prefill workgroup: 64 up to 64 rows, else 128
 
 }  // namespace w4a16

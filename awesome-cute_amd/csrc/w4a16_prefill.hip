@@ -1,12 +1,15 @@
 // Prefill W4A16 kernel (more than 64 activation rows): MFMA-bound, so the
 // design minimises everything that competes with the matrix pipe.
 //
-// One workgroup of 8 waves (two per SIMD) owns a 128-row x 256-column tile of
-// C.  Waves 0-3 run the first half of the k range and waves 4-7 the second
-// half over the same tile, and the two halves are added through LDS at the
-// end.  Two waves per SIMD matter: a wave cannot issue its own unpack/LDS
+// One workgroup of 8 waves (two per SIMD) owns a 16*RB-row x 256-column tile
+// of C (RB = 8 row blocks, or 4 when there are at most 64 rows) and, when the
+// tiles alone would leave compute units idle, one of `ksplit` slices of the k
+// range (the slices meet through the same ticketed exchange as the streaming
+// kernel's).  Waves 0-3 run the first half of the workgroup's k range and
+// waves 4-7 the second half over the same tile, and the two halves are added
+// through LDS at the end.  Two waves per SIMD matter: a wave cannot issue its own unpack/LDS
 // instructions under its own MFMAs, but the other wave's run there for free.
-// Within a half, wave w keeps a 128 x 64 fp32 accumulator (128 registers):
+// Within a half, wave w keeps a 16*RB x 64 fp32 accumulator (16*RB registers):
 // columns 16j+8h+c of the two 64-column blocks 2p, 2p+1 with p = w/2 and
 // j in {2(w%2), 2(w%2)+1}.
 //   - Weights never touch LDS: each lane reads the 8 bytes of its Marlin
@@ -43,16 +46,25 @@ namespace w4a16 {
 
 namespace {
 
-constexpr int kPfTileM = 128;
 constexpr int kPfTileN = 256;
 constexpr int kPfStageK = 64;
-constexpr int kPfStepBytes = 4 * 128 * 16 + 128;  // one 32-deep k step of the A slab (+pad)
-constexpr int kPfSlabA = 2 * kPfStepBytes;        // two steps per stage
-constexpr int kPfSlabB = 4 * 2048;                // four 16-deep rows of packed weights
-constexpr int kPfStageBytes = kPfSlabA + kPfSlabB;
-constexpr int kPfRing = 3;                        // slabs in LDS per k half
-constexpr int kPfLdsBytes = 2 * kPfRing * kPfStageBytes;
+constexpr int kPfSlabB = 4 * 2048;  // four 16-deep rows of packed weights
+constexpr int kPfRing = 3;          // slabs in LDS per k half
 constexpr int kOobPf = (int)0x80000000;
+
+// LDS geometry of a tile of RB row blocks
+template <int RB>
+struct PfShape {
+  static constexpr int kTileM = 16 * RB;
+  static constexpr int kPlane = kTileM * 16;            // one k group of a step: rows x 16 bytes
+  static constexpr int kStepBytes = 4 * kPlane + 128;   // one 32-deep k step of the A slab (+pad)
+  static constexpr int kSlabA = 2 * kStepBytes;         // two steps per stage
+  static constexpr int kStageBytes = kSlabA + kPfSlabB;
+  static constexpr int kLdsBytes = 2 * kPfRing * kStageBytes;
+  // the epilogue reuses the rings: 8 waves x RB/2 row blocks x 4 KiB of fp32
+  // to swap, then the fp16 tile with padded rows
+  static_assert(8 * (RB / 2) * 4096 <= kLdsBytes && kTileM * (kPfTileN * 2 + 16) <= kLdsBytes, "");
+};
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
@@ -60,10 +72,18 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigne
 
 }  // namespace
 
-template <bool GROUP>
-__global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, int tiles_n) {
-  extern __shared__ __attribute__((aligned(16))) char smem_all[];  // kPfLdsBytes
+template <bool GROUP, int RB>
+__global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, int tiles_n,
+                                                      int ksplit) {
+  extern __shared__ __attribute__((aligned(16))) char smem_all[];  // PfShape<RB>::kLdsBytes
+  __shared__ int s_ticket;
   W4A16_PF_TENTRY
+  constexpr int kPfTileM = PfShape<RB>::kTileM;
+  constexpr int kPlane = PfShape<RB>::kPlane;
+  constexpr int kPfStepBytes = PfShape<RB>::kStepBytes;
+  constexpr int kPfSlabA = PfShape<RB>::kSlabA;
+  constexpr int kPfStageBytes = PfShape<RB>::kStageBytes;
+  constexpr int HB = RB / 2;  // row blocks a wave finishes after the halves are added
 
   const int kh = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);  // k half
   const int tid = threadIdx.x & 255;  // thread within the half
@@ -78,9 +98,12 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a
   // contiguous run of tiles (column tile fastest) so that the workgroups
   // sharing an L2 read the same rows of A and neighbouring columns of B.
-  const int total = tiles_m * tiles_n;
-  int tile = (int)blockIdx.x;
-  if ((total & 7) == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3);
+  // The k slices of a tile are consecutive work indices, so they share an XCD.
+  const int total = tiles_m * tiles_n * ksplit;
+  int work = (int)blockIdx.x;
+  if ((total & 7) == 0) work = (work & 7) * (total >> 3) + (work >> 3);
+  const int tile = work / ksplit;
+  const int ks = work - tile * ksplit;
   const int tm = tile / tiles_n;
   const int tn = tile - tm * tiles_n;
   const int m0 = tm * kPfTileM;
@@ -109,26 +132,28 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // slab staging: thread (row = tid/8 + 32 i, chunk x = tid%8) moves 16 bytes;
   // rows past the end of A read as zeros (out-of-range buffer offset)
   const int ax = tid & 7;
-  int a_lane[4];
+  int a_lane[HB];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < HB; i++) {
     const int r = (tid >> 3) + 32 * i;
     a_lane[i] = r < rows ? r * p.K * 2 + 16 * ax : kOobPf;
   }
   // LDS slab: [step][k group][row][slot] dwords; chunk x -> step x/4, slot x%4
   const int a_wr = (ax >> 2) * kPfStepBytes + (tid >> 3) * 16 + (ax & 3) * 4;
-  const int a_rd = kg * 2048 + nu * 16;
+  const int a_rd = kg * kPlane + nu * 16;
 
   const DequantConsts dc;
   // this half's stages: [s_begin, s_end) of the K/64 stages; the loop runs the
   // same count in both halves (a stage past s_end fetches zeros)
   const int stages_all = p.K / kPfStageK;
-  const int half_stages = (stages_all + 1) >> 1;
-  const int s_begin = kh * half_stages;
-  const int s_end = kh ? stages_all : half_stages;
+  const int st0 = (int)((long long)ks * stages_all / ksplit);        // this workgroup's slice
+  const int st1 = (int)((long long)(ks + 1) * stages_all / ksplit);
+  const int half_stages = (st1 - st0 + 1) >> 1;
+  const int s_begin = st0 + kh * half_stages;
+  const int s_end = kh ? st1 : st0 + half_stages;
   const int stages = half_stages;
 
-  i4 areg[4];   // A slab of the stage after next, in flight
+  i4 areg[HB];  // A slab of the stage after next, in flight
   i4 bcopy[2];  // its packed weights
   i2 sreg[2];   // group scales of this stage and the next
 
@@ -144,7 +169,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     const int inv = sg < s_end ? 0 : kOobPf;
 #ifndef W4A16_PF_SKIP_A
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < HB; i++)
       areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
 #endif
 #ifndef W4A16_PF_SKIP_B
@@ -160,16 +185,16 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #endif
     char* base = smem + ring * kPfStageBytes;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < HB; i++)
 #pragma unroll
-      for (int g = 0; g < 4; g++) *(int*)(base + a_wr + g * 2048 + i * 32 * 16) = areg[i][g];
+      for (int g = 0; g < 4; g++) *(int*)(base + a_wr + g * kPlane + i * 32 * 16) = areg[i][g];
 #pragma unroll
     for (int i = 0; i < 2; i++) *(i4*)(base + b_wr + i * 4096) = bcopy[i];
   };
 
-  f4 acc[8][4];
+  f4 acc[RB][4];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < RB; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
@@ -177,7 +202,8 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   i4 af[4];    // ring of activation operands, three ahead of the MFMAs
   i2 bw[2];    // packed weight words of the next k step (its two 16-deep rows)
 #ifdef W4A16_PF_INIT
-  for (int i = 0; i < 4; i++) { areg[i] = (i4){tid, 1, 2, 3}; af[i] = (i4){tid, 5, 6, 7}; }
+  for (int i = 0; i < HB; i++) areg[i] = (i4){tid, 1, 2, 3};
+  for (int i = 0; i < 4; i++) af[i] = (i4){tid, 5, 6, 7};
   for (int i = 0; i < 2; i++) { bcopy[i] = (i4){tid, 9, 1, 2}; sreg[i] = (i2){tid, 3}; }
   for (int i = 0; i < 2; i++) for (int j = 0; j < 4; j++) w[i][j] = __builtin_bit_cast(h8, (i4){tid, j, i, 7});
 #endif
@@ -210,25 +236,25 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     af[idx] = *(const i4*)(step_base + a_rd + i * 256);
   };
 
-  // One 32-deep k step: 32 MFMAs on w[h] and the operand ring, while the
+  // One 32-deep k step: 4*RB MFMAs on w[h] and the operand ring, while the
   // operands of the next step are fetched from LDS and its weights unpacked
-  // into w[h^1].  `mid` runs between the fourth and fifth row block.
+  // into w[h^1].  `mid` runs half way through the row blocks.
   auto step = [&](int h, const char* cur_base, const char* nxt_base, const char* nxt_stage,
                   int nslot, int nh, auto&& mid) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < RB; i++) {
       if (i == 0) read_bw(nxt_stage, nh);
-      if (i + 3 < 8)
+      if (i + 3 < RB)
         read_frag((i + 3) & 3, cur_base, i + 3);
       else
-        read_frag((i + 3) & 3, nxt_base, i + 3 - 8);
+        read_frag((i + 3) & 3, nxt_base, i + 3 - RB);
       const h8 a = __builtin_bit_cast(h8, af[i & 3]);
 #pragma unroll
       for (int j = 0; j < 4; j++)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[h][j], a, acc[i][j], 0, 0, 0);
-      if (i == 2) dequant_pair(h ^ 1, nslot, nh, 0);
-      if (i == 3) mid();
-      if (i == 5) dequant_pair(h ^ 1, nslot, nh, 1);
+      if (i == RB / 4) dequant_pair(h ^ 1, nslot, nh, 0);
+      if (i == RB / 2 - 1) mid();
+      if (i == RB / 2 + RB / 8) dequant_pair(h ^ 1, nslot, nh, 1);
     }
   };
 
@@ -279,27 +305,81 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 
   W4A16_PF_TEND
   // ---- epilogue.  The k halves swap the row blocks they will not write
-  // (half 0 keeps blocks 0-3, half 1 keeps 4-7) through LDS and add; the slab
-  // rings are dead by now.
-  const int own = 4 * kh;  // first row block this wave finishes
+  // (half 0 keeps blocks 0..HB-1, half 1 the rest) through LDS and add; the
+  // slab rings are dead by now.
+  const int own = HB * kh;  // first row block this wave finishes
   __syncthreads();
   {
-    f4* out = (f4*)smem_all + (size_t)(kh * 4 + wave) * (16 * 64);
+    f4* out = (f4*)smem_all + (size_t)(kh * 4 + wave) * (HB * 4 * 64);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < HB; i++)
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        out[(i * 4 + j) * 64 + lane] = kh ? acc[i][j] : acc[4 + i][j];
+        out[(i * 4 + j) * 64 + lane] = kh ? acc[i][j] : acc[HB + i][j];
   }
   __syncthreads();
-  f4 fin[4][4];
+  f4 fin[HB][4];
   {
-    const f4* in = (const f4*)smem_all + (size_t)((kh ^ 1) * 4 + wave) * (16 * 64);
+    const f4* in = (const f4*)smem_all + (size_t)((kh ^ 1) * 4 + wave) * (HB * 4 * 64);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < HB; i++)
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        fin[i][j] = (kh ? acc[4 + i][j] : acc[i][j]) + in[(i * 4 + j) * 64 + lane];
+        fin[i][j] = (kh ? acc[HB + i][j] : acc[i][j]) + in[(i * 4 + j) * 64 + lane];
+  }
+
+  // ---- k slices of other workgroups.  Same exchange as the streaming
+  // kernel's: every slice writes its fp32 tile through to memory (whole 1 KiB
+  // lines per wave instruction), waits for the acknowledgement, takes the
+  // tile's ticket; the last arrival adds all slices in slice order (its own
+  // from registers at its place in that order) and carries on.  Nobody spins.
+  if (ksplit > 1) {
+    constexpr int part_bytes = kPfTileM * kPfTileN * 4;
+    const __amdgpu_buffer_rsrc_t rP = pf_rsrc(p.scratch, 0x7fffffffu);
+    const int at = ((kh * 4 + wave) * (HB * 4) * 64 + lane) * 16;
+    const int mine = work * part_bytes;
+#pragma unroll
+    for (int i = 0; i < HB; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, fin[i][j]), rP,
+                                               at + (i * 4 + j) * 1024, mine, 16 /* sc1 */);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my stores have been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0)
+      s_ticket = __hip_atomic_fetch_add(&p.locks[tile], 1, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != ksplit - 1) return;  // a later slice finishes the tile
+    f4 sum[HB][4];
+    for (int k2 = 0; k2 < ksplit; k2++) {
+      f4 v[HB][4];
+      if (k2 != ks) {
+        const int theirs = (tile * ksplit + k2) * part_bytes;
+#pragma unroll
+        for (int i = 0; i < HB; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++)
+            v[i][j] = __builtin_bit_cast(
+                f4, __builtin_amdgcn_raw_buffer_load_b128(rP, at + (i * 4 + j) * 1024, theirs,
+                                                          16 /* sc1 */));
+      } else {
+#pragma unroll
+        for (int i = 0; i < HB; i++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) v[i][j] = fin[i][j];
+      }
+#pragma unroll
+      for (int i = 0; i < HB; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) sum[i][j] = k2 == 0 ? v[i][j] : sum[i][j] + v[i][j];
+    }
+#pragma unroll
+    for (int i = 0; i < HB; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) fin[i][j] = sum[i][j];
+    if (threadIdx.x == 0)  // counters are handed back zeroed
+      __hip_atomic_store(&p.locks[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
 
@@ -318,7 +398,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       for (int r = 0; r < 4; r++) sc[r] = S[scale_index_single(kPfTileN * tn + nloc + r)];
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < HB; i++) {
       const int m = 16 * (own + i) + nu;
       h4 o = {(half_t)fin[i][j][0], (half_t)fin[i][j][1], (half_t)fin[i][j][2],
               (half_t)fin[i][j][3]};
@@ -329,7 +409,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   __syncthreads();
   half_t* C = (half_t*)p.C;
 #pragma unroll
-  for (int it = 0; it < 8; it++) {
+  for (int it = 0; it < kPfTileM / 16; it++) {
     const int piece = it * 512 + (int)threadIdx.x;  // 16-byte piece of the tile
     const int m = piece >> 5;
     const int c16 = piece & 31;
@@ -341,26 +421,37 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   W4A16_PF_TEXIT
 }
 
-int configure_prefill_kernels() {
+template <int RB>
+static int configure_rb() {
   // more LDS than the default per-workgroup limit: opt in per kernel and device
-  if (hipFuncSetAttribute((const void*)prefill_kernel<true>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess ||
-      hipFuncSetAttribute((const void*)prefill_kernel<false>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kPfLdsBytes) != hipSuccess)
+  constexpr int lds = PfShape<RB>::kLdsBytes;
+  if (hipFuncSetAttribute((const void*)prefill_kernel<true, RB>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess ||
+      hipFuncSetAttribute((const void*)prefill_kernel<false, RB>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
     return 3;
   return 0;
 }
 
-int launch_prefill(const GemmArgs& a, bool group, hipStream_t stream) {
-  const int tiles_m = ceil_div(a.M, kPfTileM);
+int configure_prefill_kernels() { return (configure_rb<8>() | configure_rb<4>()) ? 3 : 0; }
+
+template <bool GROUP, int RB>
+static void launch_rb(const GemmArgs& a, int ksplit, hipStream_t stream) {
+  const int tiles_m = ceil_div(a.M, PfShape<RB>::kTileM);
   const int tiles_n = a.N / kPfTileN;
-  const int grid = tiles_m * tiles_n;
-  if (group)
-    hipLaunchKernelGGL(prefill_kernel<true>, dim3(grid), dim3(512), kPfLdsBytes, stream, a,
-                       tiles_m, tiles_n);
-  else
-    hipLaunchKernelGGL(prefill_kernel<false>, dim3(grid), dim3(512), kPfLdsBytes, stream, a,
-                       tiles_m, tiles_n);
+  constexpr int lds = PfShape<RB>::kLdsBytes;
+  hipLaunchKernelGGL((prefill_kernel<GROUP, RB>), dim3(tiles_m * tiles_n * ksplit), dim3(512), lds,
+                     stream, a, tiles_m, tiles_n, ksplit);
+}
+
+int prefill_tile_rows(int m) { return m <= 64 ? 64 : 128; }
+
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream) {
+  if (prefill_tile_rows(a.M) == 64) {
+    if (group) launch_rb<true, 4>(a, ksplit, stream); else launch_rb<false, 4>(a, ksplit, stream);
+  } else {
+    if (group) launch_rb<true, 8>(a, ksplit, stream); else launch_rb<false, 8>(a, ksplit, stream);
+  }
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 

@@ -50,8 +50,6 @@ constexpr int kWaitVm0 = 0x0F70;
 constexpr int kAuxL2 = 1;
 constexpr int kAuxDevice = 16;
 
-typedef unsigned u4 __attribute__((ext_vector_type(4)));
-
 // 16 bytes per lane of a partial-sum slot, as whole-line buffer accesses
 template <int AUX>
 __device__ __forceinline__ void store_partial(__amdgpu_buffer_rsrc_t r, int voffset, int soffset,

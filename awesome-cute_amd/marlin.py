@@ -30,6 +30,8 @@ _lib.marlin_amd_check.restype = _I
 _lib.marlin_amd_check.argtypes = [_I] * 6
 _lib.marlin_amd_plan.restype = _I
 _lib.marlin_amd_plan.argtypes = [_I] * 8 + [_P]
+_lib.marlin_amd_force_k_slices.restype = None
+_lib.marlin_amd_force_k_slices.argtypes = [_I]
 _lib.marlin_amd_force_kernel.restype = None
 _lib.marlin_amd_force_kernel.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
@@ -202,6 +204,11 @@ def force_kernel(which):
     _lib.marlin_amd_force_kernel(int(which))
 
 
+def force_k_slices(slices):
+    """Slices of the k range per prefill tile; 0 = choose by cost (process-wide)."""
+    _lib.marlin_amd_force_k_slices(int(slices))
+
+
 def work_order(grid):
     """Work index of every workgroup of a streaming launch of `grid` workgroups."""
     out = (ctypes.c_int * grid)()
@@ -211,7 +218,8 @@ def work_order(grid):
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     """Kernel, grid and stream-K partition marlin_gemm would use."""
-    out = (ctypes.c_int * 6)()
+    out = (ctypes.c_int * 8)()
     rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
-    keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches")
+    keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
+            "k_slices", "tile_rows")
     return rc, dict(zip(keys, out))

@@ -82,7 +82,9 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * How marlin_gemm would run a problem on a device with `cus` compute units:
  * out[0] = kernel (0 = none, 1 = streaming, 2 = prefill), out[1] = workgroups,
  * out[2] = granules per workgroup (streaming), out[3] = column tiles,
- * out[4] = granules per column tile, out[5] = number of launches.
+ * out[4] = granules per column tile, out[5] = number of launches,
+ * out[6] = slices of the k range per tile (prefill), out[7] = rows of C per
+ * workgroup (prefill; 0 for the streaming kernel).  `out` holds 8 ints.
  * Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
@@ -105,6 +107,13 @@ void marlin_amd_work_order(int grid, int *out);
  * counterpart; for tests and tools.
  */
 void marlin_amd_force_kernel(int which);
+
+/*
+ * Slices of the k range per tile of the prefill kernel, process-wide: 0 =
+ * choose by cost (default), n = n slices where the problem allows (each slice
+ * at least 256 deep).  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_k_slices(int slices);
 
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *marlin_amd_last_error(void);

@@ -219,6 +219,30 @@ def test_either_kernel_above_64_rows(env, which, m):
         marlin.force_kernel(0)
 
 
+@pytest.mark.parametrize("slices", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("m", [1, 16, 40, 64, 65, 128, 200, 384])
+def test_prefill_kernel_k_slices(env, m, slices):
+    """The prefill kernel at every tile height (64 rows up to 64, else 128) and
+    with its k range cut into slices that meet through the ticketed exchange;
+    the same slicing gives the same bits every time."""
+    torch, marlin = env
+    marlin.force_kernel(2)
+    marlin.force_k_slices(slices)
+    try:
+        rc, plan = marlin.plan(m, 512, 2048, 128)
+        assert rc == 0 and plan["kernel"] == 2 and plan["k_slices"] == slices
+        assert plan["tile_rows"] == (64 if m <= 64 else 128)
+        check(env, m, 512, 2048, 128, seed=m + slices)
+        check(env, m, 256, 1024, -1, seed=m + slices + 3)  # at most 4 slices of 256
+        A, q, s, B, sp = O.make_problem(m, 768, 1536, 128, seed=5)
+        c1 = gpu_gemm(env, A, B, sp, 768)
+        c2 = gpu_gemm(env, A, B, sp, 768)
+        assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_k_slices(0)
+
+
 def test_config2_decode(env):
     check(env, 1, 4096, 4096, 128, seed=2)
 
