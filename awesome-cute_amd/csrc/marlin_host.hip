@@ -143,29 +143,11 @@ constexpr int kStreamMaxRows = 64;
 // kernel; set by marlin_amd_force_kernel (tests and tools)
 std::atomic<int> g_force_kernel{0};
 
-// Above 64 rows either kernel can do the job: the prefill kernel once, with
-// ceil(m/128) * n/256 workgroups, or the streaming kernel once per 64 rows,
-// reading the weights again every time.  Costs in us fitted to measurements
-// (n, k in {4096, 11008}, m = 64 ... 1024): a round of prefill workgroups
-// takes 6 + 0.0108 k whatever their number up to the CU count; a 64-row
-// streaming pass 11.6 + 0.52 per MB of packed weights, a last pass of at most
-// 16 rows 5 + 0.25 per MB.
-bool prefer_prefill(int m, int n, int k, int cus) {
-  const double rounds = ceil_div(ceil_div(m, 128) * (n / 256), cus);
-  const double t_prefill = rounds * (6.0 + 0.0108 * k);
-  const double mb_weights = 0.5e-6 * n * k;
-  const int tail = m % kStreamMaxRows;
-  double t_stream = (m / kStreamMaxRows) * (11.6 + 0.52 * mb_weights);
-  if (tail > 16)
-    t_stream += 11.6 + 0.52 * mb_weights;
-  else if (tail > 0)
-    t_stream += 5.0 + 0.25 * mb_weights;
-  return t_prefill <= t_stream;
-}
-
 // Slices of the k range per prefill tile.  A slice must be at least 256 deep
 // (two 64-deep stages for each half of the workgroup) and the tile counters
-// and partial-sum slots must fit; within that, 0 = by cost.
+// and partial-sum slots must fit.  Measured (m = 64 ... 1024, n, k in {4096,
+// 11008, 28672 x 8192}): filling the CUs pays up to four slices; more slices
+// only add partial-sum traffic.
 std::atomic<int> g_force_k_slices{0};
 
 int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
@@ -175,8 +157,43 @@ int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
   if (most < 1 || tiles > kMaxPrefillTiles) return 1;
   const int force = g_force_k_slices.load(std::memory_order_relaxed);
   if (force > 0) return force < most ? force : most;
-  (void)cus;
-  return 1;
+  int s = cus / tiles;
+  if (s > 4) s = 4;
+  if (s > most) s = most;
+  return s < 1 ? 1 : s;
+}
+
+// Either kernel can do any problem whose n is a multiple of 256: the prefill
+// kernel once, or the streaming kernel once per 64 rows, reading the weights
+// again every time.  Costs in us, fitted to measurements on MI355X.
+double prefill_cost(int m, int n, int k, int cus) {
+  const int tile_rows = prefill_tile_rows(m);
+  const int tiles = ceil_div(m, tile_rows) * (n / 256);
+  const int s = prefill_k_slices(tiles, tile_rows, k, cus);
+  const double rounds = ceil_div(tiles * s, cus);
+  // a full-depth tile takes 6 + 0.0108 k (two thirds of that with 64 rows)
+  // however few tiles there are; slices divide it and add their exchange
+  const double tile = (6.0 + 0.0108 * k) * (tile_rows == 64 ? 0.66 : 1.0);
+  return rounds * (tile / s + (s > 1 ? 5.0 + 2.5 * s : 0.0));
+}
+
+double stream_cost(int m, int n, int k) {
+  const double mb = 0.5e-6 * n * k;  // MB of packed weights, read once per pass
+  // a pass over 49-64 rows (4 row blocks); the slope flattens for big problems
+  const double full = mb <= 22.5 ? 11.6 + 0.52 * mb : 23.3 + 0.25 * (mb - 22.5);
+  const int tail = m % kStreamMaxRows;
+  double t = (m / kStreamMaxRows) * full;
+  if (tail > 16)
+    t += full * (tail > 48 ? 1.0 : tail > 32 ? 0.9 : 0.65);
+  else if (tail > 0)
+    t += 5.0 + 0.25 * mb;
+  return t;
+}
+
+bool prefer_prefill(int m, int n, int k, int cus) {
+  // no measurement favours 64-row prefill tiles below four row blocks
+  if (m <= 48) return false;
+  return prefill_cost(m, n, k, cus) <= stream_cost(m, n, k);
 }
 
 Plan make_plan(int m, int n, int k, int sms, int cus) {
@@ -184,8 +201,8 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   const int force = g_force_kernel.load(std::memory_order_relaxed);
   // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
   // whenever m > 16, by the shape contract)
-  const bool prefill = n % 256 == 0 && (force == 2 || (force == 0 && m > kStreamMaxRows &&
-                                                       prefer_prefill(m, n, k, cus)));
+  const bool prefill =
+      n % 256 == 0 && (force == 2 || (force == 0 && prefer_prefill(m, n, k, cus)));
   pl.ksplit = 1;
   pl.tile_rows = 0;
   if (prefill) {

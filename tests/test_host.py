@@ -33,6 +33,7 @@ def test_library_exports_every_declared_symbol(marlin):
     names = re.findall(r"\b(marlin_\w+)\s*\(", header)
     assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
             "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_force_kernel",
+            "marlin_amd_force_k_slices",
             "marlin_amd_last_error",
             "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
@@ -154,27 +155,40 @@ def test_work_order_is_an_xcd_blocked_permutation(marlin, grid):
         start += len(mine)
 
 
-def test_kernel_choice_above_64_rows(marlin):
-    """Few rows over wide weights go through the streaming kernel in 64-row
-    launches, many rows through the prefill kernel; the force knob overrides."""
-    assert marlin.plan(128, 4096, 4096, 128)[1] == {
-        **marlin.plan(64, 4096, 4096, 128)[1], "launches": 2}
-    assert marlin.plan(1024, 4096, 4096, 128)[1]["kernel"] == 2
+def test_kernel_choice_by_cost(marlin):
+    """Few rows go through the streaming kernel, many through the prefill
+    kernel, whose k range is cut into up to four slices while tiles alone would
+    leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles.  The
+    knobs override the choice."""
+    for m, n, k, kernel, slices, rows in [
+            (1, 4096, 4096, 1, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
+            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (128, 4096, 4096, 2, 4, 128),
+            (512, 4096, 4096, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
+            (2048, 4096, 4096, 2, 1, 128)]:
+        rc, p = marlin.plan(m, n, k, 128)
+        assert rc == 0 and (p["kernel"], p["k_slices"], p["tile_rows"]) == (kernel, slices, rows), \
+            (m, n, k, p)
+        if kernel == 2:
+            assert p["grid"] == -(-m // rows) * (n // 256) * slices
     try:
         marlin.force_kernel(1)
         rc, p = marlin.plan(2048, 4096, 4096, 128)
         assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32
         marlin.force_kernel(2)
         rc, p = marlin.plan(100, 512, 1024, 128)
-        assert rc == 0 and p["kernel"] == 2 and p["grid"] == 2
+        assert rc == 0 and p["kernel"] == 2 and p["grid"] == 2 * p["k_slices"]
+        marlin.force_k_slices(3)
+        assert marlin.plan(100, 512, 1024, 128)[1]["k_slices"] == 3
+        assert marlin.plan(100, 512, 512, 128)[1]["k_slices"] == 2  # slices are >= 256 deep
         assert marlin.plan(16, 128, 512, 128)[1]["kernel"] == 1  # n = 128: no 256-wide tile
     finally:
         marlin.force_kernel(0)
+        marlin.force_k_slices(0)
 
 
 def test_plan_picks_kernels(marlin):
     assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 1
-    assert marlin.plan(64, 28672, 8192, 128)[1]["kernel"] == 1
+    assert marlin.plan(32, 28672, 8192, 128)[1]["kernel"] == 1
     rc, p = marlin.plan(2048, 4096, 4096, 128)
     assert rc == 0 and p["kernel"] == 2 and p["grid"] == 16 * 16
     assert marlin.plan(16, 256, 64, -1, 128, 128)[0] == 1
