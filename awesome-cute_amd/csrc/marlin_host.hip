@@ -220,35 +220,45 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   if (sms > 0) {
     pl.sp = make_stream_plan(n, k, sms > kMaxStreamGrid ? kMaxStreamGrid : sms);
   } else {
-    // Granules per workgroup.  Measured on MI355X: a split that cuts column
-    // tiles at whole fractions (or multiples) of a tile costs about
-    // 0.1 us x row blocks per granule of the longest workgroup; a split that
-    // leaves workgroups straddling tile boundaries pays for a second fix-up
-    // per workgroup, about 1 + 2.5 x row blocks us on top.  Take the cheapest
-    // of the aligned candidates and the evenly balanced one.
+    // Measured on MI355X: a split that keeps every workgroup inside one
+    // column tile (or gives it whole tiles) costs about 0.1 us x row blocks
+    // per granule of the longest workgroup; a split that leaves workgroups
+    // straddling tile boundaries is several us slower (a second exchange per
+    // workgroup, and workgroups that read different weight rows at the same
+    // time), about 1 + 2.5 x row blocks us.  Candidates: every tile cut into
+    // c nearly equal runs (c tiles' worth of workgroups <= CUs), whole tiles
+    // per workgroup, and the evenly balanced uniform split.
     const int mb = ceil_div(m < kStreamMaxRows ? m : kStreamMaxRows, 16);
+    const int NT = n / kTileN;
     const int KG = k / kGranuleK;
-    const int total = (n / kTileN) * KG;
+    const int total = NT * KG;
     const double per_granule = 0.1 * mb, straddle = 1.0 + 2.5 * mb;
-    int best = ceil_div(total, cus);
+    int best = ceil_div(total, cus), best_wpt = 0;
     double best_cost = per_granule * best + ((best % KG == 0 || KG % best == 0) ? 0.0 : straddle);
-    auto consider = [&](int g) {
-      if (g < 1 || g > total) return;
-      const int grid = ceil_div(total, g);
-      if (grid > cus) return;  // more workgroups than CUs never paid off
+    for (int c = 1; c <= KG && NT * c <= cus; c++) {
+      const int g = ceil_div(KG, c);
       const double cost = per_granule * g;
-      if (cost < best_cost - 1e-9 || (cost < best_cost + 1e-9 && g > best)) {
+      if (cost < best_cost + 1e-9) {  // on a tie the one-tile form: its kernel is leaner
         best = g;
+        best_wpt = c;
         best_cost = cost;
       }
-    };
-    for (int d = 1; d <= KG; d++)
-      if (KG % d == 0) consider(KG / d);
-    for (int mult = 2; mult * KG <= total; mult++) consider(mult * KG);
-    pl.sp.NT = n / kTileN;
+    }
+    for (int mult = 2; mult * KG <= total; mult++) {
+      const int g = mult * KG;
+      if (ceil_div(total, g) > cus) continue;  // more workgroups than CUs never paid off
+      const double cost = per_granule * g;
+      if (cost < best_cost - 1e-9) {
+        best = g;
+        best_wpt = 0;
+        best_cost = cost;
+      }
+    }
+    pl.sp.NT = NT;
     pl.sp.KG = KG;
     pl.sp.gpb = best;
-    pl.sp.grid = ceil_div(total, best);
+    pl.sp.wpt = best_wpt;
+    pl.sp.grid = best_wpt > 0 ? NT * best_wpt : ceil_div(total, best);
   }
   pl.grid = pl.sp.grid;
   pl.launches = ceil_div(m, kStreamMaxRows);
@@ -298,6 +308,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
       a.lock_stride = 1;
       a.scratch = scratch;
       a.gpb = 0;
+      a.wpt = 0;
       rc = launch_prefill(a, groupsize != -1, pl.ksplit, stream);
       if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
     } else if (pl.kernel == 1 && scratch) {
@@ -315,6 +326,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
         a.lock_stride = lock_stride;
         a.scratch = scratch;
         a.gpb = pl.sp.gpb;
+        a.wpt = pl.sp.wpt;
         rc = launch_stream(a, groupsize != -1, pl.grid, stream);
       }
       if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
@@ -385,7 +397,7 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int* out) {
-  for (int i = 0; i < 8; i++) out[i] = 0;
+  for (int i = 0; i < 9; i++) out[i] = 0;
   int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
   Plan pl = make_plan(prob_m, prob_n, prob_k, sms, cus);
@@ -397,6 +409,7 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[5] = pl.launches;
   out[6] = pl.ksplit;
   out[7] = pl.tile_rows;
+  out[8] = pl.kernel == 1 ? pl.sp.wpt : 0;
   return rc;
 }
 

@@ -100,11 +100,17 @@ __device__ __forceinline__ unsigned pack_half2(float a, float b) {
 // with work index b owns granules [b*gpb, (b+1)*gpb).  A column tile whose granules fall into
 // more than one workgroup is finished by whichever of them arrives last at the
 // tile's counter.
+//
+// Second form (wpt > 0): every column tile is cut into wpt nearly equal runs,
+// one per workgroup: work index w owns run w % wpt of tile w / wpt.  This keeps
+// every workgroup inside one tile for any KG, where the first form can only do
+// so when gpb divides KG.
 struct StreamPlan {
   int NT;    // 128-column tiles
   int KG;    // 64-deep granules per tile
-  int gpb;   // granules per workgroup
+  int gpb;   // granules per workgroup (the most, when wpt > 0)
   int grid;  // workgroups launched (all own at least one granule)
+  int wpt;   // workgroups per tile, or 0 for the first form
 };
 
 __host__ __device__ __forceinline__ int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -118,6 +124,7 @@ __host__ __device__ inline StreamPlan make_stream_plan(int N, int K, int want_gr
   if (want_grid > total) want_grid = total;
   p.gpb = ceil_div(total, want_grid);
   p.grid = ceil_div(total, p.gpb);
+  p.wpt = 0;
   return p;
 }
 
@@ -165,7 +172,8 @@ struct GemmArgs {
   int* locks;       // N/128 counters, lock_stride ints apart; zero on entry and on exit
   int lock_stride;  // >= 1; spreads the counters over separate cache lines
   float* scratch;   // partial sums of shared tiles
-  int gpb;          // granules per workgroup (streaming kernel)
+  int gpb;          // granules per workgroup (streaming kernel; the most, when wpt > 0)
+  int wpt;          // workgroups per column tile, or 0 (see StreamPlan)
 };
 
 // bytes of fp32 partial sums of mb row blocks of 16; a slot holds them twice

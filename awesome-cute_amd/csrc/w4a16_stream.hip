@@ -125,7 +125,11 @@ __device__ __forceinline__ void lds_barrier() {
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
-template <int MB, bool GROUP, int DEPTH>
+// ONE_TILE: the plan's second form (every column tile cut into p.wpt runs), in
+// which a workgroup never leaves its tile: no tile bookkeeping in the main
+// loop and exactly one finish at the end.  Otherwise the first form (equal
+// runs of the tile-major sequence), where a run may cross tile boundaries.
+template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH>::kBytes
   __shared__ int s_ticket;
@@ -143,12 +147,24 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   plan.KG = p.K / kGranuleK;
   plan.gpb = p.gpb;
   plan.grid = (int)gridDim.x;
+  plan.wpt = ONE_TILE ? p.wpt : 0;
   const int KG = plan.KG;
   const int total = plan.NT * KG;
   const int wid = xcd_work_index((int)blockIdx.x, plan.grid);
-  const int u0 = wid * plan.gpb;
-  if (u0 >= total) return;
-  const int u1 = min(total, u0 + plan.gpb);
+  // my granules [u0, u1) of the tile-major sequence; my_tile = tile of u0
+  int u0, u1, my_tile;
+  if constexpr (ONE_TILE) {
+    my_tile = wid / p.wpt;
+    const int run = wid - my_tile * p.wpt;
+    u0 = my_tile * KG + (run * KG) / p.wpt;
+    u1 = my_tile * KG + ((run + 1) * KG) / p.wpt;
+    if (my_tile >= plan.NT || u0 >= u1) return;
+  } else {
+    u0 = wid * plan.gpb;
+    if (u0 >= total) return;
+    u1 = min(total, u0 + plan.gpb);
+    my_tile = u0 / KG;
+  }
 
   const __amdgpu_buffer_rsrc_t rB = make_rsrc(p.B, (unsigned)p.K * (unsigned)(p.N / 2));
   const __amdgpu_buffer_rsrc_t rA = make_rsrc(p.A, (unsigned)p.M * (unsigned)p.K * 2u);
@@ -343,15 +359,17 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // was anywhere else; if nobody was, the last arrival sits behind the same
     // L2 as every copy and reads those, otherwise it refetches the
     // write-through copies from memory.
-    const int bf = tile_first_block(plan, t);
-    const int bl = tile_last_block(plan, t);
+    const int bf = ONE_TILE ? t * p.wpt : tile_first_block(plan, t);
+    const int bl = ONE_TILE ? bf + p.wpt - 1 : tile_last_block(plan, t);
     bool writer = true;
     if (bl > bf) {
       // a slot is two copies of MB*4*2*64 f4: [0] written back lazily by this
       // XCD's L2, [1] written through to memory
       constexpr int part_bytes = MB * 4 * 2 * 64 * 16;
       const __amdgpu_buffer_rsrc_t rP = make_rsrc(p.scratch, 0x7fffffffu);
-      const int mine = partial_slot(plan, wid, t) * (2 * part_bytes);
+      // slot of work index b for this tile
+      auto slot_of = [&](int b) { return ONE_TILE ? 2 * b : partial_slot(plan, b, t); };
+      const int mine = slot_of(wid) * (2 * part_bytes);
       const int my_xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;  // HW_REG_XCC_ID[3:0]
       const int away = xcd_range_holds((int)blockIdx.x, (int)gridDim.x, my_xcd, bf, bl) ? 0 : 0x10000;
 #pragma unroll
@@ -388,7 +406,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
             for (int u = 0; u < 8; u++) {
               const int b = b0 + u;
               if (b <= bl && b != wid) {
-                const int theirs = partial_slot(plan, b, t) * (2 * part_bytes);
+                const int theirs = slot_of(b) * (2 * part_bytes);
                 if (same_l2) {
                   dst[u][0] = load_partial<kAuxL2>(rP, at, theirs);
                   dst[u][1] = load_partial<kAuxL2>(rP, at + 1024, theirs);
@@ -454,61 +472,72 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     }
   };
 
-  // My granules are u0 + wave, u0 + wave + 4, ... < u1, walked in one flat
-  // sequence across column tiles; (t, kq) are kept incrementally for the
-  // compute position and for the issue position DEPTH granules ahead.
+  // My granules are u0 + wave, u0 + wave + 4, ... < u1.
   const int n_mine = (u1 - u0 > wave) ? ((u1 - u0 - wave + 3) >> 2) : 0;
-  const int t_first = u0 / KG;
-  const int t_last = (u1 - 1) / KG;
-  int it = t_first, ikq = u0 - t_first * KG + wave;  // issue position
-  while (ikq >= KG) {
-    ikq -= KG;
-    ++it;
-  }
-  int ct = it, ckq = ikq;  // compute position
-  int cur_tile = t_first;  // tile whose sums are in acc
   clear_acc();
 
+  if constexpr (ONE_TILE) {
+    // one tile: the k position just advances by four granules a turn
+    int ikq = u0 - my_tile * KG + wave;  // issue position
 #pragma unroll
-  for (int d = 0; d < DEPTH; d++) {
-    issue(d, it, ikq, d < n_mine);
-    ikq += 4;
+    for (int d = 0; d < DEPTH; d++) {
+      issue(d, my_tile, ikq, d < n_mine);
+      ikq += 4;
+    }
+    W4A16_STAMP(1)
+    if constexpr (DEPTH == 2 && !kDmaA) {
+      // At most two granules per wave and both are already requested: a rolled
+      // loop over one copy of the compute code; the second granule moves into
+      // the first's registers in between.
+#pragma unroll 1
+      for (int i = 0; i < n_mine; i++) {
+        compute(0);
+        if (i == 0) { W4A16_STAMP(2) }
+#pragma unroll
+        for (int r = 0; r < 4; r++) bq[0][r] = bq[1][r];
+        sq[0] = sq[1];
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+          aq[0][m][0] = aq[1][m][0];
+          aq[0][m][1] = aq[1][m][1];
+        }
+      }
+    } else {
+      for (int base = 0; base < n_mine; base += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+          compute(d);  // a granule past the end is all zeros and adds nothing
+          if (base + d == 0) { W4A16_STAMP(2) }
+          issue(d, my_tile, ikq, base + d + DEPTH < n_mine);
+          ikq += 4;
+        }
+      }
+    }
+    finish(my_tile);
+  } else {
+    // The run is walked in one flat sequence across column tiles; (t, kq) are
+    // kept incrementally for the compute position and for the issue position
+    // DEPTH granules ahead.
+    const int t_last = (u1 - 1) / KG;
+    int it = my_tile, ikq = u0 - my_tile * KG + wave;  // issue position
     while (ikq >= KG) {
       ikq -= KG;
       ++it;
     }
-  }
+    int ct = it, ckq = ikq;  // compute position
+    int cur_tile = my_tile;  // tile whose sums are in acc
 
-  W4A16_STAMP(1)
-  if constexpr (DEPTH == 2 && !kDmaA) {
-    // At most two granules per wave and both are already requested: a rolled
-    // loop over one copy of the compute code, so that the second turn runs
-    // from the instruction cache; the second granule moves into the first's
-    // registers in between.
-#pragma unroll 1
-    for (int i = 0; i < n_mine; i++) {
-      while (cur_tile < ct) {
-        finish(cur_tile);
-        ++cur_tile;
-        clear_acc();
-      }
-      compute(0);
-      if (i == 0) { W4A16_STAMP(2) }
-      ckq += 4;
-      while (ckq >= KG) {
-        ckq -= KG;
-        ++ct;
-      }
 #pragma unroll
-      for (int r = 0; r < 4; r++) bq[0][r] = bq[1][r];
-      sq[0] = sq[1];
-#pragma unroll
-      for (int m = 0; m < MB; m++) {
-        aq[0][m][0] = aq[1][m][0];
-        aq[0][m][1] = aq[1][m][1];
+    for (int d = 0; d < DEPTH; d++) {
+      issue(d, it, ikq, d < n_mine);
+      ikq += 4;
+      while (ikq >= KG) {
+        ikq -= KG;
+        ++it;
       }
     }
-  } else {
+
+    W4A16_STAMP(1)
     for (int base = 0; base < n_mine; base += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; d++) {
@@ -536,11 +565,11 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         }
       }
     }
-  }
-  while (cur_tile <= t_last) {
-    finish(cur_tile);
-    ++cur_tile;
-    clear_acc();
+    while (cur_tile <= t_last) {
+      finish(cur_tile);
+      ++cur_tile;
+      clear_acc();
+    }
   }
   W4A16_STAMP(8)
 }
@@ -548,7 +577,12 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 template <int MB, bool GROUP, int DEPTH>
 static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
   constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
-  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH>), dim3(grid), dim3(256), lds, stream, a);
+  if (a.wpt > 0)
+    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, true>), dim3(grid), dim3(256), lds, stream,
+                       a);
+  else
+    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, false>), dim3(grid), dim3(256), lds,
+                       stream, a);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
@@ -562,8 +596,11 @@ template <int MB, bool GROUP, int DEPTH>
 static int configure_variant() {
   constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
   if (lds <= 65536) return 0;  // within the default limit of dynamic LDS
-  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH>,
-                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess
+  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, true>,
+                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
+                 hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, false>,
+                                     hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     lds) == hipSuccess
              ? 0
              : 3;
 }

@@ -218,8 +218,8 @@ def work_order(grid):
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     """Kernel, grid and stream-K partition marlin_gemm would use."""
-    out = (ctypes.c_int * 8)()
+    out = (ctypes.c_int * 9)()
     rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
     keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
-            "k_slices", "tile_rows")
+            "k_slices", "tile_rows", "wgs_per_tile")
     return rc, dict(zip(keys, out))

@@ -84,7 +84,10 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * out[2] = granules per workgroup (streaming), out[3] = column tiles,
  * out[4] = granules per column tile, out[5] = number of launches,
  * out[6] = slices of the k range per tile (prefill), out[7] = rows of C per
- * workgroup (prefill; 0 for the streaming kernel).  `out` holds 8 ints.
+ * workgroup (prefill; 0 for the streaming kernel), out[8] = workgroups per
+ * column tile when the streaming kernel cuts every tile into that many runs
+ * (then out[2] is the longest run), 0 when it cuts the tile-major sequence of
+ * granules into equal runs of out[2].  `out` holds 9 ints.
  * Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,

@@ -98,12 +98,17 @@ def test_binding_level_errors_without_gpu(marlin):
 
 def _partition(plan):
     """Re-derivation of the stream-K ownership from the plan's four numbers."""
-    NT, KG, gpb, grid = (plan[k] for k in ("col_tiles", "granules_per_tile",
-                                           "granules_per_wg", "grid"))
+    NT, KG, gpb, grid, wpt = (plan[k] for k in ("col_tiles", "granules_per_tile",
+                                                "granules_per_wg", "grid", "wgs_per_tile"))
     total = NT * KG
     owner = np.full(total, -1)
     for b in range(grid):
-        lo, hi = b * gpb, min(total, (b + 1) * gpb)
+        if wpt:  # every tile cut into wpt nearly equal runs
+            t, j = divmod(b, wpt)
+            lo, hi = t * KG + j * KG // wpt, t * KG + (j + 1) * KG // wpt
+            assert hi - lo <= gpb
+        else:    # the tile-major sequence cut into runs of gpb
+            lo, hi = b * gpb, min(total, (b + 1) * gpb)
         assert lo < hi, "every launched workgroup owns at least one granule"
         assert (owner[lo:hi] == -1).all()
         owner[lo:hi] = b
@@ -153,6 +158,29 @@ def test_work_order_is_an_xcd_blocked_permutation(marlin, grid):
         mine = [order[b] for b in range(x, grid, 8)]
         assert mine == list(range(start, start + len(mine)))
         start += len(mine)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (16, 11008, 4096), (16, 4096, 11008),
+                                   (32, 28672, 8192), (16, 256, 512), (16, 1280, 1152),
+                                   (4, 12288, 4096), (16, 4096, 10752), (8, 4096, 14336),
+                                   (48, 5120, 13824), (16, 128, 128), (16, 32768, 4096)])
+def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
+    """Without an `sms` hint the planner picks splits whose workgroups never
+    straddle a column-tile boundary (one exchange per workgroup at most) and
+    never launches more workgroups than CUs."""
+    rc, plan = marlin.plan(m, n, k, -1, -1, -1, -1, 256)
+    assert rc == 0 and plan["kernel"] == 1 and plan["grid"] <= 256
+    owner = _partition(plan)
+    KG = plan["granules_per_tile"]
+    for b in range(plan["grid"]):
+        tiles = np.unique(np.nonzero(owner == b)[0])
+        assert len(tiles) >= 1
+        if plan["wgs_per_tile"]:
+            assert len(tiles) == 1
+        else:  # whole tiles per workgroup
+            assert plan["granules_per_wg"] % KG == 0
+            for t in tiles:
+                assert (owner[t] == b).all()
 
 
 def test_kernel_choice_by_cost(marlin):
