@@ -275,6 +275,13 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   const int lock_stride = max_par < 1 ? 1 : (max_par > 16 ? 16 : max_par);
   int rc = check_shape(m, n, k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || m == 0 || n == 0 || k == 0) return rc;
+  // the kernels address A, B and C with 32-bit byte offsets
+  const long long lim = 0x7fffffffLL;
+  if ((long long)k * n / 2 > lim || (long long)m * k * 2 > lim || (long long)m * n * 2 > lim) {
+    snprintf(g_last_error, sizeof(g_last_error),
+             "operand of more than 2 GiB (m=%d n=%d k=%d): split the call", m, n, k);
+    return MARLIN_ERR_RUNTIME;
+  }
   if (dev < 0 || dev >= kMaxDevices) {
     snprintf(g_last_error, sizeof(g_last_error), "device index %d out of range", dev);
     return MARLIN_ERR_RUNTIME;

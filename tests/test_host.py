@@ -94,6 +94,11 @@ def test_binding_level_errors_without_gpu(marlin):
     # an empty problem is accepted and does nothing
     rc = f(None, None, None, None, 0, 256, 128, 1, None, 32, 0, None, -1, -1, -1, 16, 1, err, 256)
     assert rc == 0
+    # operands beyond the kernels' 32-bit byte offsets are refused before any device work
+    n, k = 65536, 131072
+    rc = f(None, None, None, None, 16, n, k, k // 128, None, n // 128 * 16, 0, None,
+           -1, -1, -1, 16, 1, err, 256)
+    assert rc == 3 and b"2 GiB" in err.value
 
 
 def _partition(plan):
