@@ -243,6 +243,28 @@ def test_prefill_kernel_k_slices(env, m, slices):
         marlin.force_k_slices(0)
 
 
+@pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
+def test_frozen_known_answers(env, tag, groupsize):
+    """The committed known answers (tests/golden): dequantised weights bit for
+    bit through one-hot rows, the GEMM inside the tolerance."""
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                             "w4a16_known_answers.npz"))
+    B, sp = g[f"{tag}_B"], g[f"{tag}_s_packed"].view(np.float16)
+    A, Cref = g[f"{tag}_A"].view(np.float16), g[f"{tag}_C"].view(np.float16)
+    K, N = A.shape[1], Cref.shape[1]
+    r = O.compare(gpu_gemm(env, A, B, sp, N), Cref)
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+    rows = list(range(0, K, 7))[:16]
+    onehot = np.zeros((len(rows), K), np.float16)
+    for i, k in enumerate(rows):
+        onehot[i, k] = 1.0
+    W = g[f"{tag}_W"].view(np.float16)
+    if groupsize == -1:
+        W = W * O.unpack_scales(sp, False)
+    assert np.array_equal(gpu_gemm(env, onehot, B, sp, N).view(np.uint16),
+                          W[rows].view(np.uint16))
+
+
 def test_config2_decode(env):
     check(env, 1, 4096, 4096, 128, seed=2)
 

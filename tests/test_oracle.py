@@ -4,6 +4,8 @@ The reference holds no golden vectors for the W4A16 path, so each oracle
 function is checked against numpy's independent fp16 arithmetic, against a
 second derivation of the same quantity, or against closed forms.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -308,3 +310,31 @@ def test_compare_helper():
     assert abs(r.rel_mean_abs_err - 0.5 / 6.5) < 1e-12
     a[0] = np.nan
     assert np.isnan(O.compare(a, b).max_abs_err)
+
+
+# ---------------------------------------------------------------- frozen known answers
+
+def _golden():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                        "w4a16_known_answers.npz")
+    return np.load(path)  # allow_pickle stays False
+
+
+@pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
+def test_oracle_reproduces_frozen_known_answers(tag, groupsize):
+    """tests/golden/w4a16_known_answers.npz (written by tests/golden/make_fixtures.py
+    from this oracle once pinned): packers, dequantiser and GEMM still give the
+    same bits."""
+    g = _golden()
+    q, s = g[f"{tag}_q"], g[f"{tag}_s"].view(np.float16)
+    K, N = q.shape
+    B = O.pack_weights(q)
+    sp = O.pack_scales(s, groupsize != -1)
+    assert np.array_equal(B, g[f"{tag}_B"])
+    assert np.array_equal(sp.view(np.uint16), g[f"{tag}_s_packed"])
+    assert np.array_equal(O.dequant(B, sp, K, N, groupsize).view(np.uint16), g[f"{tag}_W"])
+    A = g[f"{tag}_A"].view(np.float16)
+    assert np.array_equal(O.gemm(A, B, sp, N, groupsize).view(np.uint16), g[f"{tag}_C"])
+    perm, scale_perm, scale_perm_single = O.get_perms()
+    assert np.array_equal(perm, g["perm"]) and np.array_equal(scale_perm, g["scale_perm"])
+    assert np.array_equal(scale_perm_single, g["scale_perm_single"])
