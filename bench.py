@@ -9,10 +9,10 @@ in one HIP graph (kernel launches only) and bracketed by HIP events on the
 launch stream, so the host's launch cost is not part of the kernel's number;
 the eager (one host call per step) rate is reported next to it.
 
-Prints ONE JSON line: the headline workload is BASELINE config 2 (decode,
+Prints ONE JSON line: the headline workload is the decode configuration (
 M=1, N=K=4096, group 128), with `roofline` for its kernel and `cpu_baseline`
 from the CPU oracle; `shapes` carries the other points of the metric
-(M=16 and M=2048 at N=K=4096) and BASELINE configs 3 and 5, measured the same
+(M=16 and M=2048 at N=K=4096) and the MLP-pair and 64-row configurations, measured the same
 way.
 """
 import argparse
@@ -31,9 +31,9 @@ MALL_BYTES = 256 << 20
 
 SHAPES = {
     # name: (M, N, K, groupsize, bound)
-    "decode": (1, 4096, 4096, 128, "hbm"),          # BASELINE configs[1]
+    "decode": (1, 4096, 4096, 128, "hbm"),          # the configuration the metric is quoted on
     "batch16": (16, 4096, 4096, 128, "hbm"),        # metric's M=16 point
-    "prefill": (2048, 4096, 4096, 128, "mfma"),     # BASELINE configs[3]
+    "prefill": (2048, 4096, 4096, 128, "mfma"),     # the MFMA-bound configuration
     "mlp_up": (16, 11008, 4096, 128, "hbm"),        # configs[2]
     "mlp_down": (16, 4096, 11008, 128, "hbm"),
     "large_g128": (64, 28672, 8192, 128, "hbm"),    # configs[4]
@@ -181,7 +181,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--shape", default="headline",
-                    help="headline (decode, then the other BASELINE shapes) or one of: " +
+                    help="headline (decode, then the other benchmark shapes) or one of: " +
                          ", ".join(SHAPES))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -190,7 +190,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 "
-                 "(column-parallel sharding is described in DESIGN.md, not built)")
+                 "(sharding over several GPUs is not built)")
 
     import torch
     import marlin

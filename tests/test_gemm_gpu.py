@@ -90,7 +90,7 @@ def test_all_k_rows_bit_exact_through_identity(env):
 
 
 def test_config1_reference_case(env):
-    # BASELINE config 1 == first case of marlin_test.py:123-131
+    # smallest benchmark config == first case of marlin_test.py:123-131
     check(env, 16, 256, 512, 128, thread_k=128, thread_n=128)
 
 

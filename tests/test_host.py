@@ -55,7 +55,7 @@ def test_oracle_is_not_linked_into_the_product():
 
 # return codes of the reference launcher (marlin_cute_kernel.cu:39-60,95-107)
 @pytest.mark.parametrize("args,want", [
-    ((16, 256, 512, 128, -1, -1), 0),      # BASELINE config 1
+    ((16, 256, 512, 128, -1, -1), 0),      # smallest benchmark config
     ((1, 4096, 4096, 128, -1, -1), 0),
     ((2048, 4096, 4096, 128, -1, -1), 0),
     ((64, 28672, 8192, -1, -1, -1), 0),

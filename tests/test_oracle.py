@@ -265,7 +265,7 @@ def test_gemm_ref_threads_do_not_change_bits():
 
 
 def test_config1_shape_runs():
-    # BASELINE config 1: M=16, N=256, K=512, group 128 (marlin_test.py:123-131)
+    # smallest benchmark config: M=16, N=256, K=512, group 128 (marlin_test.py:123-131)
     A, q, s, B, sp = O.make_problem(16, 256, 512, 128, seed=0)
     assert B.shape == (32, 512) and sp.shape == (4, 256)
     C = O.gemm(A, B, sp, 256, 128)
