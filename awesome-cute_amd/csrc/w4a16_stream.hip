@@ -1,22 +1,24 @@
-// Streaming W4A16 kernel for at most 64 activation rows (decode and small
-// batch): the weight stream is the roofline, so every wave keeps a ring of
-// 128-bit weight loads in flight straight into registers and never waits on
+// Streaming W4A16 kernel for at most 64 activation rows per launch (decode and
+// small batch): the weight stream is the roofline, so every wave keeps a ring
+// of 128-bit weight loads in flight straight into registers and never waits on
 // another wave inside the main loop.
 //
-// Work split (see make_stream_plan): a launch is NT*KG granules of
-// 128 columns x 64 k.  A workgroup (4 waves) owns a contiguous run of
-// granules; inside a column tile its waves take granules round-robin, each
-// accumulating a private 16*MB x 128 fp32 tile.  At the end of the tile the
-// four waves are summed through LDS, and if other workgroups share the tile
-// the partial sums meet in global memory: everybody stores fp32 partials,
-// bumps the tile's counter, and the last arrival adds all partials in
-// workgroup order and writes C.  Nobody ever spins.
+// Work split (StreamPlan in w4a16_common.hpp): a launch is NT*KG granules of
+// 128 columns x 64 k in column-tile-major order.  A workgroup (4 waves) owns a
+// contiguous run of granules -- one of wpt runs of a single tile, or an equal
+// share of the whole sequence -- chosen by its work index, which follows the
+// XCD the hardware deals the workgroup to (xcd_work_index).  Its waves take
+// the granules round-robin, each accumulating a private 16*MB x 128 fp32
+// tile.  At the end of a tile the four waves are summed through LDS, and if
+// other workgroups share the tile the partial sums meet in global memory:
+// everybody stores fp32 partials, bumps the tile's counter, and the last
+// arrival adds all partials in workgroup order and writes C.  Nobody spins.
 //
 // All global reads are buffer loads issued unconditionally, DEPTH granules
 // ahead, so that the hardware's in-order load counter can be waited on
 // exactly; a granule that does not exist is requested at an out-of-range
-// offset, which returns zeros without touching memory.  The ring keeps
-// running across column tiles: the first granules of the next tile are in
+// offset, which returns zeros without touching memory.  Where a run crosses
+// tiles the ring keeps running: the first granules of the next tile are in
 // flight while the current tile is reduced and written.
 #include "w4a16_common.hpp"
 
