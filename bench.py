@@ -199,7 +199,7 @@ def main():
         sys.exit("bench.py: no GPU visible")
 
     if args.shape == "headline":
-        main_name, others = "decode", ["batch16", "prefill", "mlp_up", "mlp_down", "large_g128"]
+        main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128"]
     else:
         main_name, others = args.shape, []
 
@@ -207,7 +207,7 @@ def main():
         # keep the captured graph and the run time bounded for the big shapes
         M, N, K, g, _ = SHAPES[name]
         gflop = 2.0 * M * N * K / 1e9
-        cap = 2000 if gflop < 2 else (400 if gflop < 40 else 100)
+        cap = 2000 if gflop < 2 else 400
         return max(1, min(args.steps, cap)) if name != main_name else args.steps
 
     if args.copy_calibration:
