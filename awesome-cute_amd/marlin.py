@@ -5,6 +5,7 @@ no fallback path, and a missing library is an import-time error.
 """
 import ctypes
 import os
+import threading
 
 import numpy as np
 import torch
@@ -51,21 +52,51 @@ def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16, cut
     Asynchronous on the current stream of A's device.  Raises RuntimeError where
     the reference binding raises (marlin_gemm.cpp:27-31,48-55).
     """
-    for name, t in (("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)):
-        if not t.is_cuda:
-            raise RuntimeError(f"{name} must be a GPU tensor")
-        if not t.is_contiguous():
-            raise RuntimeError(f"{name} must be contiguous")
+    if not (A.is_cuda and B.is_cuda and C.is_cuda and s.is_cuda and workspace.is_cuda):
+        _complain((("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)), "is_cuda",
+                  "must be a GPU tensor")
+    if not (A.is_contiguous() and B.is_contiguous() and C.is_contiguous() and s.is_contiguous()
+            and workspace.is_contiguous()):
+        _complain((("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)),
+                  "is_contiguous", "must be contiguous")
     dev = A.get_device()
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    err = ctypes.create_string_buffer(512)
+    err = _errbuf()
     rc = _lib.marlin_mul(A.data_ptr(), B.data_ptr(), C.data_ptr(), s.data_ptr(),
                          A.size(0), C.size(1), A.size(1), s.size(0),
-                         workspace.data_ptr(), workspace.numel(), dev, stream,
-                         thread_k, thread_n, sms, max_par, int(bool(cute_version)),
-                         err, len(err))
+                         workspace.data_ptr(), workspace.numel(), dev, _raw_stream(dev),
+                         thread_k, thread_n, sms, max_par, 1 if cute_version else 0,
+                         err, 512)
     if rc != 0:
         raise RuntimeError(err.value.decode() or f"marlin_mul failed with code {rc}")
+
+
+def _complain(named, attr, what):
+    for name, t in named:
+        v = getattr(t, attr)
+        if not (v() if callable(v) else v):
+            raise RuntimeError(f"{name} {what}")
+
+
+# The host side of a call matters at one row (the kernel takes 6.5 us): the
+# error buffer is kept per thread, and the current stream is read through
+# torch's raw-handle accessor where this torch build has it.
+_tls = threading.local()
+
+
+def _errbuf():
+    buf = getattr(_tls, "err", None)
+    if buf is None:
+        buf = _tls.err = ctypes.create_string_buffer(512)
+    return buf
+
+
+_get_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _raw_stream(dev):
+    if _get_raw_stream is not None:
+        return _get_raw_stream(dev)
+    return torch.cuda.current_stream(dev).cuda_stream
 
 
 # ---------------------------------------------------------------------------
