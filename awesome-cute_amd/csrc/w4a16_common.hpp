@@ -131,23 +131,13 @@ __host__ __device__ inline StreamPlan make_stream_plan(int N, int K, int want_gr
 // The hardware deals workgroups to the 8 XCDs round-robin (blockIdx % 8) and
 // every XCD has an L2 of its own.  Workgroup blockIdx takes the work index
 // below, so that consecutive work indices (the sharers of a column tile) sit
-// behind one L2.  This is a placement hint only: the kernel checks the XCD it
-// really runs on before it trusts a line of that L2.
+// behind one L2 and read the same activation and scale lines through it
+// (measured: up to 1 us per launch at 16 rows).  A placement hint only:
+// nothing depends on where a workgroup really runs.
 __host__ __device__ __forceinline__ int xcd_work_index(int block, int grid) {
   const int x = block & 7, q = grid >> 3, rem = grid & 7;
   return x * q + (x < rem ? x : rem) + (block >> 3);
 }
-// True if `block` runs on the XCD the round-robin dealing predicts (xcd is
-// the one it really runs on) and that XCD's run of work indices holds all of
-// [first, last].
-__host__ __device__ __forceinline__ bool xcd_range_holds(int block, int grid, int xcd, int first,
-                                                         int last) {
-  const int x = block & 7, q = grid >> 3, rem = grid & 7;
-  const int lo = x * q + (x < rem ? x : rem);
-  const int hi = lo + q + (x < rem ? 1 : 0);
-  return xcd == x && first >= lo && last < hi;
-}
-
 // first / last workgroup (by work index) touching tile t
 __host__ __device__ __forceinline__ int tile_first_block(const StreamPlan& p, int t) {
   return (t * p.KG) / p.gpb;
@@ -176,11 +166,8 @@ struct GemmArgs {
   int wpt;          // workgroups per column tile, or 0 (see StreamPlan)
 };
 
-// bytes of fp32 partial sums of mb row blocks of 16; a slot holds them twice
-// (a write-back copy for readers behind the same L2, a write-through copy for
-// everybody else)
-constexpr size_t stream_partial_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
-constexpr size_t stream_slot_bytes(int mb) { return 2 * stream_partial_bytes(mb); }
+// bytes of fp32 partial sums of mb row blocks of 16 (one slot)
+constexpr size_t stream_slot_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
 
 // Per-device set-up of the kernels that need more dynamic LDS than the default
 // limit; call once with the device current before the first launch on it.
