@@ -169,9 +169,8 @@ def test_workspace_stride_follows_max_par(env, max_par):
 
 
 def test_back_to_back_launches_share_scratch(env):
-    """Launches on one stream reuse the partial-sum slots (and the copies of
-    them that an XCD's L2 keeps): different inputs of one shape, and then
-    another shape, must not see each other's partial sums."""
+    """Launches on one stream reuse the partial-sum slots: different inputs of
+    one shape, and then another shape, must not see each other's partial sums."""
     torch, marlin = env
     dev = torch.device("cuda:0")
     probs = [O.make_problem(m, n, k, 128, seed) for (m, n, k, seed) in
