@@ -38,6 +38,9 @@ SHAPES = {
     "mlp_down": (16, 4096, 11008, 128, "hbm"),
     "large_g128": (64, 28672, 8192, 128, "hbm"),    # configs[4]
     "large_chan": (64, 28672, 8192, -1, "hbm"),
+    # not one of the benchmark's configurations: the decode kernel where the
+    # launch and exchange latencies are small beside the weight stream
+    "decode_large": (1, 28672, 8192, 128, "hbm"),
 }
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE /
@@ -199,7 +202,8 @@ def main():
         sys.exit("bench.py: no GPU visible")
 
     if args.shape == "headline":
-        main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128"]
+        main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128",
+                                        "decode_large"]
     else:
         main_name, others = args.shape, []
 
