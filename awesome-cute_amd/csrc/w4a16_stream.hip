@@ -66,12 +66,19 @@ __device__ __forceinline__ f4 load_partial(__amdgpu_buffer_rsrc_t r, int voffset
 // slot, so the activations are loaded straight into an LDS ring instead
 // (buffer_load ... lds, 16 bytes per lane) and never occupy a register before
 // they are an MFMA operand.
-template <int MB, int DEPTH>
+template <int MB, int DEPTH, bool ONE_TILE>
 struct StreamLds {
   static constexpr bool kDmaA = MB >= 2;
   static constexpr int kReduceBytes = 32768;
   static constexpr int kRingBytesPerWave = kDmaA ? DEPTH * MB * 2048 : 0;
-  static constexpr int kBytes = kReduceBytes + 4 * kRingBytesPerWave;
+  // A workgroup that stays inside one tile reduces only once, after its last
+  // granule, when the ring is dead: the reduction then reuses the ring's
+  // memory, which leaves room for a deeper ring.
+  static constexpr bool kAliased = ONE_TILE && kDmaA;
+  static constexpr int kRingBase = kAliased ? 0 : kReduceBytes;
+  static constexpr int kBytes =
+      kAliased ? (4 * kRingBytesPerWave > kReduceBytes ? 4 * kRingBytesPerWave : kReduceBytes)
+               : kReduceBytes + 4 * kRingBytesPerWave;
 };
 
 // 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at
@@ -127,9 +134,10 @@ constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (
 // runs of the tile-major sequence), where a run may cross tile boundaries.
 template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH>::kBytes
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH, ONE_TILE>::kBytes
   __shared__ int s_ticket;
-  constexpr bool kDmaA = StreamLds<MB, DEPTH>::kDmaA;
+  using Lds = StreamLds<MB, DEPTH, ONE_TILE>;
+  constexpr bool kDmaA = Lds::kDmaA;
 
   W4A16_STAMP_DECL
   const int tid = threadIdx.x;
@@ -187,15 +195,14 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     r = r < p.M ? r : p.M - 1;  // rows past M are never written back
     a_lane[i] = r * p.K * 2 + 16 * ax;
   }
-  char* lds_a = kDmaA ? smem + StreamLds<MB, DEPTH>::kReduceBytes +
-                            wave * StreamLds<MB, DEPTH>::kRingBytesPerWave
+  char* lds_a = kDmaA ? smem + Lds::kRingBase + wave * Lds::kRingBytesPerWave
                       : smem + wave * (MB * 2048);
   const int a_wr = ((lane >> 2) * 4 + ax) * 4;
   const int a_rd = kDmaA ? 16 * nu + 4 * kg : (kg * 16 + nu) * 16;
   if constexpr (kDmaA) {
     // A granule that does not exist multiplies zero weights with whatever its
     // ring slot holds, so the ring must never hold NaN or Inf bit patterns.
-    for (int o = lane * 16; o < StreamLds<MB, DEPTH>::kRingBytesPerWave; o += 1024)
+    for (int o = lane * 16; o < Lds::kRingBytesPerWave; o += 1024)
       *(i4*)(lds_a + o) = (i4){0, 0, 0, 0};
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): zeros are in before the first ring load
   }
@@ -324,6 +331,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // (j = w, h = 0/1) of every row block
     f4 res[MB][2];
     W4A16_STAMP(3)
+    // where the reduction reuses the ring's memory, the (empty) ring loads still
+    // in flight must have landed before anybody writes there
+    if constexpr (Lds::kAliased) __builtin_amdgcn_s_waitcnt(kWaitVm0);
     lds_barrier();
     W4A16_STAMP(4)
 #pragma unroll
@@ -556,41 +566,32 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   W4A16_STAMP(8)
 }
 
-template <int MB, bool GROUP, int DEPTH>
-static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
-  constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
-  if (a.wpt > 0)
-    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, true>), dim3(grid), dim3(256), lds, stream,
-                       a);
-  else
-    hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, false>), dim3(grid), dim3(256), lds,
-                       stream, a);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
-}
-
-// ring depth of the deep variant of each row-block count
-template <int MB>
+// ring depth of the deep variant: a workgroup inside one tile can afford four
+// slots for any row-block count (see StreamLds), the other form three from
+// three row blocks on
+template <int MB, bool ONE_TILE>
 constexpr int deep_ring() {
-  return MB <= 2 ? 4 : 3;
+  return (ONE_TILE || MB <= 2) ? 4 : 3;
 }
 
-template <int MB, bool GROUP, int DEPTH>
+template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
 static int configure_variant() {
-  constexpr int lds = StreamLds<MB, DEPTH>::kBytes;
+  constexpr int lds = StreamLds<MB, DEPTH, ONE_TILE>::kBytes;
   if (lds <= 65536) return 0;  // within the default limit of dynamic LDS
-  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, true>,
-                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess &&
-                 hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, false>,
-                                     hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     lds) == hipSuccess
+  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, ONE_TILE>,
+                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess
              ? 0
              : 3;
 }
+template <int MB, bool ONE_TILE>
+static int configure_form() {
+  return configure_variant<MB, false, 2, ONE_TILE>() | configure_variant<MB, true, 2, ONE_TILE>() |
+         configure_variant<MB, false, deep_ring<MB, ONE_TILE>(), ONE_TILE>() |
+         configure_variant<MB, true, deep_ring<MB, ONE_TILE>(), ONE_TILE>();
+}
 template <int MB>
 static int configure_row_blocks() {
-  return configure_variant<MB, false, 2>() | configure_variant<MB, true, 2>() |
-         configure_variant<MB, false, deep_ring<MB>()>() |
-         configure_variant<MB, true, deep_ring<MB>()>();
+  return configure_form<MB, false>() | configure_form<MB, true>();
 }
 
 int configure_stream_kernels() {
@@ -600,12 +601,26 @@ int configure_stream_kernels() {
              : 0;
 }
 
-template <int MB, bool GROUP>
-static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
+template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
+static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
+  constexpr int lds = StreamLds<MB, DEPTH, ONE_TILE>::kBytes;
+  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE>), dim3(grid), dim3(256), lds,
+                     stream, a);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+template <int MB, bool GROUP, bool ONE_TILE>
+static int launch_form(const GemmArgs& a, int grid, hipStream_t stream) {
   // ring depth: shallow when a wave only ever sees a couple of granules
   const int per_wave = (a.gpb + 3) / 4;
-  if (per_wave <= 2) return launch_variant<MB, GROUP, 2>(a, grid, stream);
-  return launch_variant<MB, GROUP, deep_ring<MB>()>(a, grid, stream);
+  if (per_wave <= 2) return launch_variant<MB, GROUP, 2, ONE_TILE>(a, grid, stream);
+  return launch_variant<MB, GROUP, deep_ring<MB, ONE_TILE>(), ONE_TILE>(a, grid, stream);
+}
+
+template <int MB, bool GROUP>
+static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
+  return a.wpt > 0 ? launch_form<MB, GROUP, true>(a, grid, stream)
+                   : launch_form<MB, GROUP, false>(a, grid, stream);
 }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream) {
