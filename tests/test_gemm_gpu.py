@@ -369,3 +369,15 @@ def test_layer_forward_matches_oracle(env):
                       groupsize)
         r = O.compare(out.cpu().numpy().reshape(m, n), Cref)
         assert r.max_abs_err <= TOL * r.max_abs_ref
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_profiling_row(env, groupsize):
+    """One case of the LLaMA sweep harness at a small size: it checks the result
+    against torch's fp32 product itself and reports both times."""
+    import marlin_profiling as mp
+    print(f"  run_profiling m=16 n=512 k=1024 group={groupsize}", flush=True)
+    row = mp.run_profiling(16, 512, 1024, groupsize, iters=5, model="t")
+    assert row['shape(m_n_k_group)'] == f"t_16_512_1024_{groupsize}"
+    assert float(row['resident_us']) > 0 and float(row['hbm_us']) > 0
+    assert float(row['max_rel_err']) <= TOL

@@ -305,3 +305,31 @@ def test_mul_refuses_cpu_tensors(marlin):
     A = torch.zeros((1, 128), dtype=torch.half)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         marlin.mul(A, A, A, A, A)
+
+
+def test_profiling_sweep_shapes_are_accepted(marlin):
+    """The sweep's layer table is the reference's (marlin_profiling.py:88-113) and
+    every case of it passes the shape contract."""
+    import marlin_profiling as mp
+    assert mp.MODELS['7B'] == [(4096, 12288), (4096, 4096), (4096, 21504), (10752, 4096)]
+    assert mp.MODELS['70B'][2:] == [(8192, 43520), (21760, 8192)]
+    assert len(mp.MODELS) == 4 and all(len(v) == 4 for v in mp.MODELS.values())
+    for layers in mp.MODELS.values():
+        for k, n in layers:
+            for g in mp.GROUP_SIZES:
+                for m in mp.BATCHES:
+                    assert marlin.check(m, n, k, g) == 0, (m, n, k, g)
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_profiling_gen_quant4_on_cpu(marlin, groupsize):
+    """gen_quant4 of the sweep: the packed buffers decode (through the oracle's
+    unpackers) to a weight equal to the fake-quantised one it returns."""
+    import marlin_profiling as mp
+    k, n = 256, 128
+    ref, B, sp = mp.gen_quant4(k, n, groupsize, dev='cpu', seed=1)
+    q = O.unpack_weights(B.numpy(), k, n)
+    s = O.unpack_scales(sp.numpy(), groupsize != -1)
+    gs = k if groupsize == -1 else groupsize
+    want = (q.astype(np.float32) - 8).astype(np.float16) * np.repeat(s, gs, axis=0)
+    assert np.array_equal(want.view(np.uint16), ref.numpy().view(np.uint16))
