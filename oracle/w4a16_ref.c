@@ -191,6 +191,8 @@ void marlin_weight_coord(int kt, int word, int e, int *k, int *n) {
 
 void marlin_unpack_weights(const int32_t *B, int K, int N, uint8_t *q) {
   int words = 2 * N;
+  /* rows kt write disjoint rows of q */
+#pragma omp parallel for schedule(static)
   for (int kt = 0; kt < K / 16; kt++)
     for (int w = 0; w < words; w++) {
       uint32_t word = (uint32_t)B[(size_t)kt * words + w];
@@ -247,10 +249,12 @@ void w4a16_dequant_ref(const int32_t *B, const uint16_t *sp, int K, int N,
                        int groupsize, uint16_t *W) {
   uint8_t *q = (uint8_t *)malloc((size_t)K * N);
   marlin_unpack_weights(B, K, N, q);
+  uint16_t zp[16]; /* fp16(q - 8): small integers, exact */
+  for (int i = 0; i < 16; i++) zp[i] = ref_f32_to_f16((float)(i - 8));
 #pragma omp parallel for schedule(static)
   for (int k = 0; k < K; k++) {
     for (int n = 0; n < N; n++) {
-      uint16_t v = ref_f32_to_f16((float)((int)q[(size_t)k * N + n] - 8));
+      uint16_t v = zp[q[(size_t)k * N + n]];
       if (groupsize > 0) {
         int g = k / groupsize;
         uint16_t s = sp[(size_t)g * N + marlin_scale_index_group(n)];
