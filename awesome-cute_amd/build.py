@@ -12,6 +12,7 @@ SOURCES = {
     "marlin_host.hip": [],
     "w4a16_stream.hip": [],
     "w4a16_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "f16_streamk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -1,0 +1,512 @@
+// Dense fp16 GEMM with a stream-K tail for gfx950: C (m x n, row-major) =
+// A (m x k, row-major) * B^T with B given as n rows of k ("TN": both operands
+// k-contiguous), fp32 accumulation, alpha = 1, beta = 0 -- the problem of the
+// reference's gemm/streamk_gemm (gemm_streamk.cu:8-110), with the same split
+// of the output tiles into a data-parallel part and a stream-K part
+// (dp_sk_block.h:82-128, strategy sk1tile_dp): tiles that fill whole waves of
+// compute units are computed by one workgroup each; the tiles of the last,
+// partial wave are cut along k into slices, one workgroup per slice, and the
+// slices of a tile meet through fp32 partial sums in memory and a counter.
+// Unlike the reference's turnstile (gemm_streamk.h:562-590: every block waits
+// for the one before it) nobody waits: a slice writes its partial tile through
+// to memory, takes a ticket, and the last arrival adds all slices in slice
+// order and writes C.
+//
+// Kernel: a workgroup of 8 waves (2 x 4, two per SIMD) owns a 256 x 256 tile
+// of C; a wave holds a 128 x 64 fp32 accumulator (128 registers).  With B as
+// the first MFMA operand and A as the second, v_mfma_f32_16x16x32_f16 yields
+// D[n][m]; lane l = 16kg + nu of an operand holds k = 8kg ... 8kg+7 of row nu.
+// Per 32-deep k stage the workgroup brings a 256 x 32 slab of A and of B into
+// a ring of four LDS slabs with buffer loads that write LDS directly (16
+// bytes per lane, lane l at 16*l): lane (kg, nu) fetches bytes [16kg, 16kg+16)
+// of the 64-byte k run of row nu, so a 16-row block is 1 KiB in [kg][row]
+// order and an operand is one conflict-free ds_read_b128.  Slabs are
+// requested two stages ahead; one barrier per stage.  The compiler cannot
+// know which slab a load in flight writes, so the LDS reads of the main loop
+// and their waits are written by hand (LDS reads return in order).
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <mutex>
+#include <type_traits>
+#include <vector>
+
+#include "../../include/streamk_amd.h"
+#include "w4a16_common.hpp"
+
+namespace w4a16 {
+
+namespace {
+
+constexpr int kDnTile = 256;     // rows and columns of a tile of C
+constexpr int kDnStageK = 32;    // k depth of a stage (one MFMA k step)
+constexpr int kDnRing = 4;       // slabs in LDS
+constexpr int kDnSlabA = 16 * 1024;
+constexpr int kDnSlab = 32 * 1024;
+constexpr int kDnLds = kDnRing * kDnSlab;
+constexpr int kDnOob = (int)0x80000000;
+constexpr int kDnPartBytes = kDnTile * kDnTile * 4;  // fp32 partial sums of one slice
+constexpr int kDnMaxSlots = 256;                     // slices in flight per launch
+constexpr int kDnMaxSlices = 4;
+
+struct DenseArgs {
+  const void* A;
+  const void* B;
+  void* C;
+  int M, N, K;
+  int tiles_n;
+  int dp_tiles;  // tiles computed by one workgroup each
+  int sk_tiles;  // tiles (the last ones in tile order) cut into ksplit slices
+  int ksplit;
+  int* locks;      // one zeroed counter per stream-K tile, zero again afterwards
+  float* scratch;  // kDnPartBytes per slice
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t dn_rsrc(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+
+// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at
+// dst + 16*l (dst is wave-uniform).  The instruction's immediate offset stays
+// zero: the hardware would add it to the LDS address as well.  (Device pass
+// only; the host pass just needs the kernel's launch stub.)
+__device__ __forceinline__ void dn_dma16(__amdgpu_buffer_rsrc_t rsrc, char* dst, int voffset,
+                                         int soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr)dst, 16, voffset, soffset, 0, 0);
+#endif
+}
+
+// LDS reads of the main loop, outside the compiler's dependence tracking
+template <int OFF>
+__device__ __forceinline__ void dn_read16(unsigned at, i4& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(OFF) : "memory");
+#endif
+}
+// wait until at most PENDING later LDS reads are outstanding; `v` is the
+// operand the wait is for
+template <int PENDING>
+__device__ __forceinline__ void dn_wait(i4& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
+#endif
+}
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
+constexpr int dn_vmcnt(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
+}  // namespace
+
+__global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // kDnLds
+  __shared__ int s_ticket;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int kg = lane >> 4;
+  const int nu = lane & 15;
+  const int wm = wave >> 2;  // 128-row half of the tile
+  const int wn = wave & 3;   // 64-column quarter
+
+  // stream-K slices come first in the grid, so that they run beside the first
+  // wave of whole tiles
+  const int sk_blocks = p.sk_tiles * p.ksplit;
+  const int work = (int)blockIdx.x;
+  int tile, ks, ksplit;
+  if (work < sk_blocks) {
+    tile = p.dp_tiles + work / p.ksplit;
+    ks = work % p.ksplit;
+    ksplit = p.ksplit;
+  } else {
+    tile = work - sk_blocks;
+    ks = 0;
+    ksplit = 1;
+  }
+  const int tm = tile / p.tiles_n;
+  const int tn = tile - tm * p.tiles_n;
+  const int m0 = tm * kDnTile;
+  const int n0 = tn * kDnTile;
+  const int rows = min(kDnTile, p.M - m0);
+
+  const __amdgpu_buffer_rsrc_t rA =
+      dn_rsrc((const char*)p.A + (size_t)m0 * p.K * 2, (unsigned)rows * (unsigned)p.K * 2u);
+  const __amdgpu_buffer_rsrc_t rB =
+      dn_rsrc((const char*)p.B + (size_t)n0 * p.K * 2, (unsigned)kDnTile * (unsigned)p.K * 2u);
+
+  // wave w fetches 16-row blocks 2w, 2w+1 of the A slab and of the B slab;
+  // rows past the end of A repeat the last row (never stored)
+  int a_src[2], b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = 16 * (2 * wave + i) + nu;
+    a_src[i] = (r < rows ? r : rows - 1) * p.K * 2 + 16 * kg;
+    b_src[i] = r * p.K * 2 + 16 * kg;
+  }
+  // this workgroup's stages [st0, st1) of the K/32 stages
+  const int stages_all = p.K / kDnStageK;
+  const int st0 = (int)((long long)ks * stages_all / ksplit);
+  const int st1 = (int)((long long)(ks + 1) * stages_all / ksplit);
+  const int stages = st1 - st0;
+
+  auto issue_slab = [&](int s, int ring) {
+    const int inv = s < stages ? 0 : kDnOob;  // a stage past the end fetches zeros
+    const int at = (st0 + s) * (kDnStageK * 2);
+    char* base = smem + ring * kDnSlab;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      dn_dma16(rA, base + (2 * wave + i) * 1024, a_src[i] | inv, at);
+      dn_dma16(rB, base + kDnSlabA + (2 * wave + i) * 1024, b_src[i] | inv, at);
+    }
+  };
+
+  f4 acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  i4 w[2][4];  // B operands of the current and the next stage
+  i4 af[4];    // ring of A operands, three ahead of the MFMAs
+  const unsigned a_rd = (unsigned)(size_t)smem + 256 * kg + 16 * nu + 8 * wm * 1024;
+  const unsigned b_rd = (unsigned)(size_t)smem + kDnSlabA + 256 * kg + 16 * nu + 4 * wn * 1024;
+
+  // prologue: slabs 0, 1, 2 requested; slab 0 landed; its first operands read
+  issue_slab(0, 0);
+  issue_slab(1, 1);
+  issue_slab(2, 2);
+  __builtin_amdgcn_s_waitcnt(dn_vmcnt(8));
+  __builtin_amdgcn_s_barrier();
+  dn_read16<0>(b_rd, w[0][0]);
+  dn_read16<1024>(b_rd, w[0][1]);
+  dn_read16<2048>(b_rd, w[0][2]);
+  dn_read16<3072>(b_rd, w[0][3]);
+  dn_read16<0>(a_rd, af[0]);
+  dn_read16<1024>(a_rd, af[1]);
+  dn_read16<2048>(a_rd, af[2]);
+
+  // One stage (H = which of the two operand buffers holds its B operands).
+  // LDS reads in issue order: ... A0' A1' A2' | B0..B3 (next stage) A3 | A4 |
+  // ... | A7 | A0'' | A1'' | A2'' with primes the prefetches of the stage
+  // before and after; when row block i is used, the reads issued after Ai may
+  // still be pending: three A operands, plus the four B reads while i < 3.
+  auto stage = [&](auto H, unsigned cur, unsigned nxt) {
+    constexpr int h = decltype(H)::value;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if (i == 0) {
+        dn_read16<0>(b_rd + nxt, w[h ^ 1][0]);
+        dn_read16<1024>(b_rd + nxt, w[h ^ 1][1]);
+        dn_read16<2048>(b_rd + nxt, w[h ^ 1][2]);
+        dn_read16<3072>(b_rd + nxt, w[h ^ 1][3]);
+      }
+      switch (i) {  // i is a constant after unrolling
+        case 0: dn_read16<3 * 1024>(a_rd + cur, af[3]); break;
+        case 1: dn_read16<4 * 1024>(a_rd + cur, af[0]); break;
+        case 2: dn_read16<5 * 1024>(a_rd + cur, af[1]); break;
+        case 3: dn_read16<6 * 1024>(a_rd + cur, af[2]); break;
+        case 4: dn_read16<7 * 1024>(a_rd + cur, af[3]); break;
+        case 5: dn_read16<0 * 1024>(a_rd + nxt, af[0]); break;
+        case 6: dn_read16<1 * 1024>(a_rd + nxt, af[1]); break;
+        case 7: dn_read16<2 * 1024>(a_rd + nxt, af[2]); break;
+      }
+      if (i < 3)
+        dn_wait<7>(af[i & 3]);
+      else
+        dn_wait<3>(af[i & 3]);
+      if (i == 0) {
+        // the B operands of this stage were requested before A0 was
+#pragma unroll
+        for (int j = 0; j < 4; j++) asm volatile("" : "+v"(w[h][j]));
+      }
+      const h8 a = __builtin_bit_cast(h8, af[i & 3]);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, w[h][j]), a,
+                                                           acc[i][j], 0, 0, 0);
+    }
+  };
+
+  int ring = 0;  // slab of the stage being computed
+  for (int s = 0; s < stages; s += 2) {
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int cs = s + u;
+      const int ring_next = (ring + 1) & (kDnRing - 1);
+      // Slab cs+1 (requested two stages ago) must have landed for every wave
+      // before this stage prefetches from it; only the four loads of slab cs+2
+      // may still be in flight.  The slab that stage cs+3 goes into was last
+      // read in stage cs-1, which every wave has left once past the barrier.
+      __builtin_amdgcn_s_waitcnt(dn_vmcnt(4));
+      __builtin_amdgcn_s_barrier();
+      issue_slab(cs + 3, (ring + 3) & (kDnRing - 1));
+      if (u == 0)
+        stage(std::integral_constant<int, 0>{}, ring * kDnSlab, ring_next * kDnSlab);
+      else
+        stage(std::integral_constant<int, 1>{}, ring * kDnSlab, ring_next * kDnSlab);
+      ring = ring_next;
+    }
+  }
+  // The loop runs an even number of stages; an odd slice computes one stage of
+  // zeros.  Nothing of the ring may still be on its way when LDS is reused.
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  // ---- slices of other workgroups: every slice writes its fp32 tile through
+  // to memory (whole 1 KiB lines per wave instruction), waits for the
+  // acknowledgement and takes the tile's ticket; the last arrival adds all
+  // slices in slice order (its own from registers at its place in that order).
+  if (ksplit > 1) {
+    const __amdgpu_buffer_rsrc_t rP = dn_rsrc(p.scratch, 0x7fffffffu);
+    const int at = (wave * 32 * 64 + lane) * 16;
+    const int mine = work * kDnPartBytes;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, acc[i][j]), rP,
+                                               at + (i * 4 + j) * 1024, mine, 16 /* sc1 */);
+    __builtin_amdgcn_s_waitcnt(dn_vmcnt(0));  // my stores have been acknowledged
+    __syncthreads();
+    const int sk_tile = tile - p.dp_tiles;
+    if (tid == 0)
+      s_ticket = __hip_atomic_fetch_add(&p.locks[sk_tile], 1, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != ksplit - 1) return;  // a later slice finishes the tile
+    // one row block at a time: the other slices' values are requested
+    // together, then added in slice order with my own at its place
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      f4 v[kDnMaxSlices][4];
+#pragma unroll
+      for (int k2 = 0; k2 < kDnMaxSlices; k2++) {
+        const int theirs = (sk_tile * ksplit + k2) * kDnPartBytes;
+        const int inv = (k2 < ksplit && k2 != ks) ? 0 : kDnOob;  // no traffic for the rest
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          v[k2][j] = __builtin_bit_cast(
+              f4, __builtin_amdgcn_raw_buffer_load_b128(rP, (at + (i * 4 + j) * 1024) | inv,
+                                                        theirs, 16 /* sc1 */));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        f4 sum = (ks == 0) ? acc[i][j] : v[0][j];
+#pragma unroll
+        for (int k2 = 1; k2 < kDnMaxSlices; k2++)
+          if (k2 < ksplit) sum += (k2 == ks) ? acc[i][j] : v[k2][j];
+        acc[i][j] = sum;
+      }
+    }
+    if (tid == 0)  // counters are handed back zeroed
+      __hip_atomic_store(&p.locks[sk_tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // ---- C: lane holds, per (i, j), row 16i + nu and four consecutive columns
+  half_t* C = (half_t*)p.C;
+  const int q = lane >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int m = 128 * wm + 16 * i + nu;
+    if (m < rows) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int n = n0 + 64 * wn + 16 * j + 4 * q;
+        const h4 o = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2],
+                      (half_t)acc[i][j][3]};
+        *(h4*)(C + (size_t)(m0 + m) * p.N + n) = o;
+      }
+    }
+  }
+}
+
+}  // namespace w4a16
+
+// ---------------------------------------------------------------------------
+// Host side: the tile split, the scratch for partial sums, the C ABI.
+
+namespace {
+
+using namespace w4a16;
+
+constexpr int kDnMaxDevices = 16;
+constexpr size_t kDnPartialBytes = (size_t)kDnMaxSlots * kDnPartBytes;
+constexpr size_t kDnScratchBytes = kDnPartialBytes + (size_t)kDnMaxSlots * sizeof(int);
+
+thread_local char g_dn_error[256] = "";
+
+void dn_set_error(hipError_t e, const char* what) {
+  snprintf(g_dn_error, sizeof(g_dn_error), "%s: %s", what, hipGetErrorString(e));
+}
+
+// one buffer of partial sums and tile counters per (device, stream), kept
+// until the process ends; the counters are zero whenever no launch is in flight
+struct DnScratch {
+  hipStream_t stream;
+  float* ptr;
+};
+struct DnDevice {
+  int cus = 0;
+  bool configured = false;
+  std::vector<DnScratch> scratch;
+};
+std::mutex g_dn_mu;
+DnDevice g_dn[kDnMaxDevices];
+
+struct DnPlan {
+  int tiles_m, tiles_n, dp_tiles, sk_tiles, ksplit, grid;
+};
+
+// Whole waves of tiles go to one workgroup each; the tiles of the partial last
+// wave are cut into as many k slices as there are idle compute units per tile
+// (at most four: beyond that the partial-sum traffic of the one workgroup that
+// finishes a tile costs more than the slices save), each at least 256 deep.
+DnPlan dn_plan(int m, int n, int k, int cus) {
+  DnPlan pl;
+  pl.tiles_m = ceil_div(m, kDnTile);
+  pl.tiles_n = n / kDnTile;
+  const int tiles = pl.tiles_m * pl.tiles_n;
+  const int rem = cus > 0 ? tiles % cus : 0;
+  int s = 1;
+  if (rem > 0) {
+    s = cus / rem;
+    if (s > kDnMaxSlices) s = kDnMaxSlices;
+    if (s > k / 256) s = k / 256;
+    while (s > 1 && rem * s > kDnMaxSlots) --s;
+    if (s < 1) s = 1;
+  }
+  pl.ksplit = s;
+  pl.sk_tiles = s > 1 ? rem : 0;
+  pl.dp_tiles = tiles - pl.sk_tiles;
+  pl.grid = pl.dp_tiles + pl.sk_tiles * s;
+  return pl;
+}
+
+int dn_check(int m, int n, int k) {
+  if (m < 0 || n < 0 || k < 0) return STREAMK_ERR_SHAPE;
+  if (n % kDnTile != 0 || k % kDnStageK != 0) return STREAMK_ERR_SHAPE;
+  return STREAMK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, int dev,
+                    void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  int rc = dn_check(m, n, k);
+  if (rc != STREAMK_OK || m == 0 || n == 0) return rc;
+  if (k == 0) {  // an empty sum
+    hipError_t e = hipMemsetAsync(C, 0, (size_t)m * n * 2, stream);
+    if (e != hipSuccess) {
+      dn_set_error(e, "hipMemsetAsync");
+      return STREAMK_ERR_RUNTIME;
+    }
+    return STREAMK_OK;
+  }
+  // a tile's rows of A and of B are addressed with 32-bit byte offsets
+  if ((long long)kDnTile * k * 2 > 0x7fffffffLL) {
+    snprintf(g_dn_error, sizeof(g_dn_error), "k = %d is too deep for 32-bit tile offsets", k);
+    return STREAMK_ERR_RUNTIME;
+  }
+  if (dev < 0 || dev >= kDnMaxDevices) {
+    snprintf(g_dn_error, sizeof(g_dn_error), "device index %d out of range", dev);
+    return STREAMK_ERR_RUNTIME;
+  }
+  int prev = -1;
+  hipError_t e = hipGetDevice(&prev);
+  if (e != hipSuccess) {
+    dn_set_error(e, "hipGetDevice");
+    return STREAMK_ERR_RUNTIME;
+  }
+  if (prev != dev && (e = hipSetDevice(dev)) != hipSuccess) {
+    dn_set_error(e, "hipSetDevice");
+    return STREAMK_ERR_RUNTIME;
+  }
+  rc = STREAMK_ERR_RUNTIME;
+  do {
+    float* scratch = nullptr;
+    int cus = 0;
+    {
+      std::lock_guard<std::mutex> lk(g_dn_mu);
+      DnDevice& d = g_dn[dev];
+      if (d.cus == 0) {
+        e = hipDeviceGetAttribute(&d.cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) {
+          d.cus = 0;
+          dn_set_error(e, "hipDeviceGetAttribute");
+          break;
+        }
+      }
+      cus = d.cus;
+      if (!d.configured) {
+        e = hipFuncSetAttribute((const void*)dense_kernel,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kDnLds);
+        if (e != hipSuccess) {
+          dn_set_error(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+          break;
+        }
+        d.configured = true;
+      }
+      for (const DnScratch& s : d.scratch)
+        if (s.stream == stream) scratch = s.ptr;
+      if (!scratch) {
+        e = hipMalloc((void**)&scratch, kDnScratchBytes);
+        if (e != hipSuccess) {
+          dn_set_error(e, "hipMalloc(scratch)");
+          break;
+        }
+        e = hipMemset((char*)scratch + kDnPartialBytes, 0, kDnScratchBytes - kDnPartialBytes);
+        if (e != hipSuccess) {
+          dn_set_error(e, "hipMemset(scratch)");
+          (void)hipFree(scratch);
+          break;
+        }
+        d.scratch.push_back({stream, scratch});
+      }
+    }
+    const DnPlan pl = dn_plan(m, n, k, cus);
+    DenseArgs a;
+    a.A = A;
+    a.B = B;
+    a.C = C;
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.tiles_n = pl.tiles_n;
+    a.dp_tiles = pl.dp_tiles;
+    a.sk_tiles = pl.sk_tiles;
+    a.ksplit = pl.ksplit;
+    a.locks = (int*)((char*)scratch + kDnPartialBytes);
+    a.scratch = scratch;
+    hipLaunchKernelGGL(dense_kernel, dim3(pl.grid), dim3(512), kDnLds, stream, a);
+    e = hipGetLastError();
+    if (e != hipSuccess) {
+      dn_set_error(e, "kernel launch");
+      break;
+    }
+    rc = STREAMK_OK;
+  } while (false);
+  if (prev != dev) (void)hipSetDevice(prev);
+  return rc;
+}
+
+int streamk_amd_check(int m, int n, int k) { return dn_check(m, n, k); }
+
+int streamk_amd_plan(int m, int n, int k, int cus, int* out) {
+  const int rc = dn_check(m, n, k);
+  if (rc != STREAMK_OK) return rc;
+  const DnPlan pl = dn_plan(m, n, k, cus);
+  out[0] = pl.tiles_m;
+  out[1] = pl.tiles_n;
+  out[2] = pl.dp_tiles;
+  out[3] = pl.sk_tiles;
+  out[4] = pl.ksplit;
+  out[5] = pl.grid;
+  return STREAMK_OK;
+}
+
+const char* streamk_amd_last_error(void) { return g_dn_error; }
+
+}  // extern "C"

@@ -390,6 +390,43 @@ void gen_quant4_ref(const uint16_t *w, int K, int N, int groupsize,
     }
 }
 
+/* ------------------------------------------------ dense fp16 GEMM ("TN") */
+
+/* C[m][n] = fp16( sum_k A[m][k] * B[n][k] ), fp32 accumulation in ascending k:
+ * the problem of the reference's gemm/streamk_gemm (gemm_streamk.cu:27-33,
+ * A row-major, B column-major k x n = n rows of k, alpha 1, beta 0). */
+int f16_gemm_tn_ref(const uint16_t *A, const uint16_t *B, uint16_t *C, int M,
+                    int N, int K, int threads) {
+  if (M <= 0 || N <= 0) return 0;
+#ifdef _OPENMP
+  omp_set_num_threads(threads > 0 ? threads : omp_get_max_threads());
+#else
+  (void)threads;
+#endif
+  float *Af = (float *)malloc((size_t)M * (K > 0 ? K : 1) * 4);
+  float *Bf = (float *)malloc((size_t)N * (K > 0 ? K : 1) * 4);
+  if (!Af || !Bf) {
+    free(Af);
+    free(Bf);
+    return -1;
+  }
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)M * K; i++) Af[i] = ref_f16_to_f32(A[i]);
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)N * K; i++) Bf[i] = ref_f16_to_f32(B[i]);
+#pragma omp parallel for schedule(dynamic, 16) collapse(2)
+  for (int m = 0; m < M; m++)
+    for (int n = 0; n < N; n++) {
+      const float *a = Af + (size_t)m * K, *b = Bf + (size_t)n * K;
+      float acc = 0.0f;
+      for (int k = 0; k < K; k++) acc += a[k] * b[k];
+      C[(size_t)m * N + n] = ref_f32_to_f16(acc);
+    }
+  free(Af);
+  free(Bf);
+  return 0;
+}
+
 /* -------------------------------------------------------------- comparison */
 
 void w4a16_compare(const uint16_t *C, const uint16_t *Cref, size_t n,

@@ -97,6 +97,12 @@ void w4a16_dequant_ref(const int32_t *B, const uint16_t *sp, int K, int N,
 int w4a16_gemm_ref(const uint16_t *A, const int32_t *B, const uint16_t *sp,
                    uint16_t *C, int M, int N, int K, int groupsize,
                    int threads);
+/* Dense fp16 GEMM of the sibling path gemm/streamk_gemm: C (M x N) =
+ * A (M x K, row-major) * B^T with B as N rows of K; fp32 accumulation in
+ * ascending k, one rounding to fp16.  Pinned against numpy's float64 matmul
+ * (tests/test_streamk_host.py).  Returns 0, or -1 without memory. */
+int f16_gemm_tn_ref(const uint16_t *A, const uint16_t *B, uint16_t *C, int M,
+                    int N, int K, int threads);
 /* Same result type, float64 accumulation straight from the packed nibbles
  * through marlin_weight_coord; O(MNK) scalar, for tiny shapes only. */
 void w4a16_gemm_ref_f64(const uint16_t *A, const int32_t *B,

@@ -44,6 +44,8 @@ def _load():
     lib.gen_quant4_ref.argtypes = [P, c.c_int, c.c_int, c.c_int, P, P, P]
     lib.w4a16_compare.argtypes = [P, P, c.c_size_t, P]
     lib.w4a16_ref_max_threads.restype = c.c_int
+    lib.f16_gemm_tn_ref.restype = c.c_int
+    lib.f16_gemm_tn_ref.argtypes = [P, P, P] + [c.c_int] * 4
     return lib
 
 
@@ -108,6 +110,19 @@ def gemm(A, B, sp, N, groupsize, threads=0):
     M, K = A.shape
     C = np.zeros((M, N), np.uint16)
     rc = lib.w4a16_gemm_ref(_p(A), _p(B), _p(sp), _p(C), M, N, K, groupsize, threads)
+    assert rc == 0
+    return C.view(np.float16)
+
+
+def dense_gemm_tn(A, B, threads=0):
+    """A (M, K) and B (N, K) float16 -> C (M, N) float16, fp32 accumulation."""
+    A = np.ascontiguousarray(A).view(np.uint16)
+    B = np.ascontiguousarray(B).view(np.uint16)
+    M, K = A.shape
+    N = B.shape[0]
+    assert B.shape[1] == K
+    C = np.zeros((M, N), np.uint16)
+    rc = lib.f16_gemm_tn_ref(_p(A), _p(B), _p(C), M, N, K, threads)
     assert rc == 0
     return C.view(np.float16)
 
