@@ -16,14 +16,19 @@
 // of C; a wave holds a 128 x 64 fp32 accumulator (128 registers).  With B as
 // the first MFMA operand and A as the second, v_mfma_f32_16x16x32_f16 yields
 // D[n][m]; lane l = 16kg + nu of an operand holds k = 8kg ... 8kg+7 of row nu.
-// Per 32-deep k stage the workgroup brings a 256 x 32 slab of A and of B into
-// a ring of four LDS slabs with buffer loads that write LDS directly (16
-// bytes per lane, lane l at 16*l): lane (kg, nu) fetches bytes [16kg, 16kg+16)
-// of the 64-byte k run of row nu, so a 16-row block is 1 KiB in [kg][row]
-// order and an operand is one conflict-free ds_read_b128.  Slabs are
-// requested two stages ahead; one barrier per stage.  The compiler cannot
-// know which slab a load in flight writes, so the LDS reads of the main loop
-// and their waits are written by hand (LDS reads return in order).
+// Per 64-deep k stage (two MFMA k steps) the workgroup brings a 256 x 64 slab
+// of A and of B into one of two LDS slabs with buffer loads that write LDS
+// directly (16 bytes per lane, lane l at 16*l).  Eight lanes fetch the whole
+// 128-byte k run of a row -- one cache line; with 64-byte runs every line
+// came in twice and the loads alone bounded the kernel -- so a slab is
+// row-major with 128-byte rows.  To keep the operand reads (lane (kg, nu):
+// 16 bytes at chunk 4h + kg of row nu, one ds_read_b128) free of bank
+// conflicts, the chunk stored at position c of row r is chunk c ^ (r % 8);
+// since the hardware fixes where a lane's bytes land, the swizzle is applied
+// to the address the lane fetches.  A slab is requested a whole stage before
+// it is needed; one barrier per stage.  The compiler cannot know which slab a
+// load in flight writes, so the LDS reads of the main loop and their waits are
+// written by hand (LDS reads return in order).
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -39,10 +44,10 @@ namespace w4a16 {
 namespace {
 
 constexpr int kDnTile = 256;     // rows and columns of a tile of C
-constexpr int kDnStageK = 32;    // k depth of a stage (one MFMA k step)
-constexpr int kDnRing = 4;       // slabs in LDS
-constexpr int kDnSlabA = 16 * 1024;
-constexpr int kDnSlab = 32 * 1024;
+constexpr int kDnStageK = 64;    // k depth of a stage (two MFMA k steps)
+constexpr int kDnRing = 2;       // slabs in LDS
+constexpr int kDnSlabA = 32 * 1024;
+constexpr int kDnSlab = 64 * 1024;
 constexpr int kDnLds = kDnRing * kDnSlab;
 constexpr int kDnOob = (int)0x80000000;
 constexpr int kDnPartBytes = kDnTile * kDnTile * 4;  // fp32 partial sums of one slice
@@ -134,16 +139,21 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   const __amdgpu_buffer_rsrc_t rB =
       dn_rsrc((const char*)p.B + (size_t)n0 * p.K * 2, (unsigned)kDnTile * (unsigned)p.K * 2u);
 
-  // wave w fetches 16-row blocks 2w, 2w+1 of the A slab and of the B slab;
-  // rows past the end of A repeat the last row (never stored)
-  int a_src[2], b_src[2];
+  // wave w fetches rows 32w ... 32w+31 of the A slab and of the B slab, eight
+  // rows per instruction: lane (r = lane/8, c = lane%8) lands at [r][c] and
+  // fetches chunk c ^ r of its row.  Rows past the end of A repeat the last
+  // row (never stored).
+  int a_src[4], b_src[4];
+  {
+    const int r8 = lane >> 3, c = (lane & 7) ^ r8;
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int r = 16 * (2 * wave + i) + nu;
-    a_src[i] = (r < rows ? r : rows - 1) * p.K * 2 + 16 * kg;
-    b_src[i] = r * p.K * 2 + 16 * kg;
+    for (int t = 0; t < 4; t++) {
+      const int r = 32 * wave + 8 * t + r8;
+      a_src[t] = (r < rows ? r : rows - 1) * p.K * 2 + 16 * c;
+      b_src[t] = r * p.K * 2 + 16 * c;
+    }
   }
-  // this workgroup's stages [st0, st1) of the K/32 stages
+  // this workgroup's stages [st0, st1) of the K/64 stages
   const int stages_all = p.K / kDnStageK;
   const int st0 = (int)((long long)ks * stages_all / ksplit);
   const int st1 = (int)((long long)(ks + 1) * stages_all / ksplit);
@@ -152,11 +162,11 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   auto issue_slab = [&](int s, int ring) {
     const int inv = s < stages ? 0 : kDnOob;  // a stage past the end fetches zeros
     const int at = (st0 + s) * (kDnStageK * 2);
-    char* base = smem + ring * kDnSlab;
+    char* base = smem + ring * kDnSlab + (32 * wave) * 128;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-      dn_dma16(rA, base + (2 * wave + i) * 1024, a_src[i] | inv, at);
-      dn_dma16(rB, base + kDnSlabA + (2 * wave + i) * 1024, b_src[i] | inv, at);
+    for (int t = 0; t < 4; t++) {
+      dn_dma16(rA, base + t * 1024, a_src[t] | inv, at);
+      dn_dma16(rB, base + kDnSlabA + t * 1024, b_src[t] | inv, at);
     }
   };
 
@@ -166,56 +176,76 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
-  i4 w[2][4];  // B operands of the current and the next stage
+  i4 w[2][4];  // B operands of the two k steps of a stage
   i4 af[4];    // ring of A operands, three ahead of the MFMAs
-  const unsigned a_rd = (unsigned)(size_t)smem + 256 * kg + 16 * nu + 8 * wm * 1024;
-  const unsigned b_rd = (unsigned)(size_t)smem + kDnSlabA + 256 * kg + 16 * nu + 4 * wn * 1024;
+  // operand addresses in slab 0 for the two k steps
+  unsigned a_rd[2], b_rd[2];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const unsigned sw = 16 * ((4 * h + kg) ^ (nu & 7));
+    a_rd[h] = (unsigned)(size_t)smem + (128 * wm + nu) * 128 + sw;
+    b_rd[h] = (unsigned)(size_t)smem + kDnSlabA + (64 * wn + nu) * 128 + sw;
+  }
 
-  // prologue: slabs 0, 1, 2 requested; slab 0 landed; its first operands read
+  // prologue: slabs 0 and 1 requested; slab 0 landed; its first operands read
   issue_slab(0, 0);
   issue_slab(1, 1);
-  issue_slab(2, 2);
   __builtin_amdgcn_s_waitcnt(dn_vmcnt(8));
   __builtin_amdgcn_s_barrier();
-  dn_read16<0>(b_rd, w[0][0]);
-  dn_read16<1024>(b_rd, w[0][1]);
-  dn_read16<2048>(b_rd, w[0][2]);
-  dn_read16<3072>(b_rd, w[0][3]);
-  dn_read16<0>(a_rd, af[0]);
-  dn_read16<1024>(a_rd, af[1]);
-  dn_read16<2048>(a_rd, af[2]);
+  dn_read16<0>(b_rd[0], w[0][0]);
+  dn_read16<2048>(b_rd[0], w[0][1]);
+  dn_read16<4096>(b_rd[0], w[0][2]);
+  dn_read16<6144>(b_rd[0], w[0][3]);
+  dn_read16<0>(a_rd[0], af[0]);
+  dn_read16<2048>(a_rd[0], af[1]);
+  dn_read16<4096>(a_rd[0], af[2]);
 
-  // One stage (H = which of the two operand buffers holds its B operands).
-  // LDS reads in issue order: ... A0' A1' A2' | B0..B3 (next stage) A3 | A4 |
-  // ... | A7 | A0'' | A1'' | A2'' with primes the prefetches of the stage
-  // before and after; when row block i is used, the reads issued after Ai may
-  // still be pending: three A operands, plus the four B reads while i < 3.
-  auto stage = [&](auto H, unsigned cur, unsigned nxt) {
+  // One k step (H) of the stage in slab `cur`.  LDS reads in issue order, with
+  // Ai the operand of row block i and primes the prefetches for the step after:
+  //   step 0:  | B(step 1) x4  A3 | A4 | A5 | A6 | A7 | A0' | A1' | A2' |
+  //   step 1:  | A3 | A4 | A5 | A6 | A7 | barrier, B(next stage) x4  A0' | A1' | A2' |
+  // When row block i is used, the reads issued after Ai may still be pending:
+  // three A operands, plus the four B reads where those were issued in between.
+  // The barrier of a stage sits where the first read from the next slab is
+  // about to be issued: by then every wave has its own part of that slab (it
+  // waits for its loads first) and has issued and received all its reads of
+  // the current slab, which the request for the stage after next overwrites.
+  auto kstep = [&](auto H, unsigned cur, unsigned nxt, int s) {
     constexpr int h = decltype(H)::value;
+    const unsigned ac = a_rd[h] + cur;                        // this step, this slab
+    const unsigned an = h ? a_rd[0] + nxt : a_rd[1] + cur;    // the step after
+    const unsigned bn = h ? b_rd[0] + nxt : b_rd[1] + cur;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      if (i == 0) {
-        dn_read16<0>(b_rd + nxt, w[h ^ 1][0]);
-        dn_read16<1024>(b_rd + nxt, w[h ^ 1][1]);
-        dn_read16<2048>(b_rd + nxt, w[h ^ 1][2]);
-        dn_read16<3072>(b_rd + nxt, w[h ^ 1][3]);
+      if ((h == 0 && i == 0) || (h == 1 && i == 5)) {
+        if (h == 1) {
+          __builtin_amdgcn_s_waitcnt(0);  // my loads of the next slab and my reads of this one
+          __builtin_amdgcn_s_barrier();
+#ifndef DN_SKIP_LOADS
+          issue_slab(s + 2, (int)(cur != 0));
+#endif
+        }
+        dn_read16<0>(bn, w[h ^ 1][0]);
+        dn_read16<2048>(bn, w[h ^ 1][1]);
+        dn_read16<4096>(bn, w[h ^ 1][2]);
+        dn_read16<6144>(bn, w[h ^ 1][3]);
       }
       switch (i) {  // i is a constant after unrolling
-        case 0: dn_read16<3 * 1024>(a_rd + cur, af[3]); break;
-        case 1: dn_read16<4 * 1024>(a_rd + cur, af[0]); break;
-        case 2: dn_read16<5 * 1024>(a_rd + cur, af[1]); break;
-        case 3: dn_read16<6 * 1024>(a_rd + cur, af[2]); break;
-        case 4: dn_read16<7 * 1024>(a_rd + cur, af[3]); break;
-        case 5: dn_read16<0 * 1024>(a_rd + nxt, af[0]); break;
-        case 6: dn_read16<1 * 1024>(a_rd + nxt, af[1]); break;
-        case 7: dn_read16<2 * 1024>(a_rd + nxt, af[2]); break;
+        case 0: dn_read16<3 * 2048>(ac, af[3]); break;
+        case 1: dn_read16<4 * 2048>(ac, af[0]); break;
+        case 2: dn_read16<5 * 2048>(ac, af[1]); break;
+        case 3: dn_read16<6 * 2048>(ac, af[2]); break;
+        case 4: dn_read16<7 * 2048>(ac, af[3]); break;
+        case 5: dn_read16<0 * 2048>(an, af[0]); break;
+        case 6: dn_read16<1 * 2048>(an, af[1]); break;
+        case 7: dn_read16<2 * 2048>(an, af[2]); break;
       }
-      if (i < 3)
+      if ((h == 0 && i < 3) || (h == 1 && i >= 5))
         dn_wait<7>(af[i & 3]);
       else
         dn_wait<3>(af[i & 3]);
       if (i == 0) {
-        // the B operands of this stage were requested before A0 was
+        // the B operands of this step were requested before A0 was
 #pragma unroll
         for (int j = 0; j < 4; j++) asm volatile("" : "+v"(w[h][j]));
       }
@@ -227,28 +257,12 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     }
   };
 
-  int ring = 0;  // slab of the stage being computed
-  for (int s = 0; s < stages; s += 2) {
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-      const int cs = s + u;
-      const int ring_next = (ring + 1) & (kDnRing - 1);
-      // Slab cs+1 (requested two stages ago) must have landed for every wave
-      // before this stage prefetches from it; only the four loads of slab cs+2
-      // may still be in flight.  The slab that stage cs+3 goes into was last
-      // read in stage cs-1, which every wave has left once past the barrier.
-      __builtin_amdgcn_s_waitcnt(dn_vmcnt(4));
-      __builtin_amdgcn_s_barrier();
-      issue_slab(cs + 3, (ring + 3) & (kDnRing - 1));
-      if (u == 0)
-        stage(std::integral_constant<int, 0>{}, ring * kDnSlab, ring_next * kDnSlab);
-      else
-        stage(std::integral_constant<int, 1>{}, ring * kDnSlab, ring_next * kDnSlab);
-      ring = ring_next;
-    }
+  for (int s = 0; s < stages; s++) {
+    const unsigned cur = (s & 1) ? kDnSlab : 0, nxt = (s & 1) ? 0 : kDnSlab;
+    kstep(std::integral_constant<int, 0>{}, cur, nxt, s);
+    kstep(std::integral_constant<int, 1>{}, cur, nxt, s);
   }
-  // The loop runs an even number of stages; an odd slice computes one stage of
-  // zeros.  Nothing of the ring may still be on its way when LDS is reused.
+  // Nothing of the ring may still be on its way when LDS is reused.
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 

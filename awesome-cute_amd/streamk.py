@@ -55,7 +55,7 @@ def gemm(A, B, C=None):
     rc = _lib.streamk_gemm_tn(A.data_ptr(), B.data_ptr(), C.data_ptr(), m, n, k, dev, stream)
     if rc == 1:
         raise ValueError(f"shape (m={m}, n={n}, k={k}) not supported: n must be a multiple of 256, "
-                         "k of 32")
+                         "k of 64")
     if rc != 0:
         raise RuntimeError("streamk_gemm_tn: " + _lib.streamk_amd_last_error().decode())
     return C

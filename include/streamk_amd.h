@@ -17,13 +17,13 @@ extern "C" {
 #endif
 
 #define STREAMK_OK 0
-#define STREAMK_ERR_SHAPE 1   /* negative size, n not a multiple of 256, k not a multiple of 32 */
+#define STREAMK_ERR_SHAPE 1   /* negative size, n not a multiple of 256, k not a multiple of 64 */
 #define STREAMK_ERR_RUNTIME 3 /* HIP error or size limit; text in streamk_amd_last_error() */
 
 /* C = A * B^T on `hip_stream` (a hipStream_t) of device `dev`; asynchronous.
  * A: m x k fp16, row-major.  B: n x k fp16, row-major (the k x n column-major
  * operand of gemm_streamk.cu:29).  C: m x n fp16, row-major, written once.
- * fp32 accumulation.  m is arbitrary; n % 256 == 0 and k % 32 == 0.
+ * fp32 accumulation.  m is arbitrary; n % 256 == 0 and k % 64 == 0.
  * Partial sums of the stream-K tiles live in a library-owned buffer (64 MiB +
  * 1 KiB of counters per (device, stream), allocated on the first call on a
  * stream and kept): calls on one stream may follow each other freely, calls
