@@ -59,13 +59,29 @@ struct DenseArgs {
   const void* B;
   void* C;
   int M, N, K;
-  int tiles_n;
+  int tiles_m, tiles_n;
   int dp_tiles;  // tiles computed by one workgroup each
   int sk_tiles;  // tiles (the last ones in tile order) cut into ksplit slices
   int ksplit;
   int* locks;      // one zeroed counter per stream-K tile, zero again afterwards
   float* scratch;  // kDnPartBytes per slice
 };
+
+// Tiles are numbered panel by panel: a panel is kDnPanel column tiles wide
+// (the last one narrower), and inside a panel the column tile runs fastest.
+// A run of consecutive tile numbers then covers a compact block of C, so the
+// workgroups that share an L2 read few distinct rows of A and B.
+constexpr int kDnPanel = 8;
+__host__ __device__ __forceinline__ void dn_tile_coord(int t, int tiles_m, int tiles_n, int* tm,
+                                                       int* tn) {
+  const int per_panel = tiles_m * kDnPanel;
+  const int p = t / per_panel;
+  const int first = p * kDnPanel;
+  const int width = tiles_n - first < kDnPanel ? tiles_n - first : kDnPanel;
+  const int o = t - p * per_panel;
+  *tm = o / width;
+  *tn = first + o - *tm * width;
+}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t dn_rsrc(const void* p, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
@@ -124,12 +140,15 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     ks = work % p.ksplit;
     ksplit = p.ksplit;
   } else {
+    // The hardware deals workgroups to the 8 XCDs round-robin; give every XCD
+    // a contiguous run of tile numbers.  A placement hint only.
     tile = work - sk_blocks;
+    if (((sk_blocks | p.dp_tiles) & 7) == 0) tile = (tile & 7) * (p.dp_tiles >> 3) + (tile >> 3);
     ks = 0;
     ksplit = 1;
   }
-  const int tm = tile / p.tiles_n;
-  const int tn = tile - tm * p.tiles_n;
+  int tm, tn;
+  dn_tile_coord(tile, p.tiles_m, p.tiles_n, &tm, &tn);
   const int m0 = tm * kDnTile;
   const int n0 = tn * kDnTile;
   const int rows = min(kDnTile, p.M - m0);
@@ -488,6 +507,7 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.M = m;
     a.N = n;
     a.K = k;
+    a.tiles_m = pl.tiles_m;
     a.tiles_n = pl.tiles_n;
     a.dp_tiles = pl.dp_tiles;
     a.sk_tiles = pl.sk_tiles;
@@ -519,6 +539,10 @@ int streamk_amd_plan(int m, int n, int k, int cus, int* out) {
   out[4] = pl.ksplit;
   out[5] = pl.grid;
   return STREAMK_OK;
+}
+
+void streamk_amd_tile_coord(int tile, int tiles_m, int tiles_n, int* out) {
+  dn_tile_coord(tile, tiles_m, tiles_n, &out[0], &out[1]);
 }
 
 const char* streamk_amd_last_error(void) { return g_dn_error; }

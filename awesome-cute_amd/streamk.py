@@ -21,6 +21,8 @@ _lib.streamk_amd_check.restype = _I
 _lib.streamk_amd_check.argtypes = [_I, _I, _I]
 _lib.streamk_amd_plan.restype = _I
 _lib.streamk_amd_plan.argtypes = [_I, _I, _I, _I, _P]
+_lib.streamk_amd_tile_coord.restype = None
+_lib.streamk_amd_tile_coord.argtypes = [_I, _I, _I, _P]
 _lib.streamk_amd_last_error.restype = ctypes.c_char_p
 
 
@@ -35,6 +37,13 @@ def plan(m, n, k, cus=256):
     rc = _lib.streamk_amd_plan(m, n, k, cus, out)
     keys = ("tiles_m", "tiles_n", "dp_tiles", "sk_tiles", "k_slices", "grid")
     return rc, dict(zip(keys, out))
+
+
+def tile_coord(tile, tiles_m, tiles_n):
+    """(row tile, column tile) of a tile number."""
+    out = (ctypes.c_int * 2)()
+    _lib.streamk_amd_tile_coord(tile, tiles_m, tiles_n, out)
+    return out[0], out[1]
 
 
 def gemm(A, B, C=None):

@@ -36,9 +36,13 @@ int streamk_amd_check(int m, int n, int k);
 
 /* the tile split for a device with `cus` compute units (counterpart of
  * SK_DP_Block_Wrapper, dp_sk_block.h:31-80): out[0..5] = tiles along m, tiles
- * along n (256 x 256 tiles, column tile fastest), data-parallel tiles, stream-K
+ * along n (256 x 256 tiles, numbered in panels of 8 column tiles), data-parallel tiles, stream-K
  * tiles (the last ones in tile order), k slices per stream-K tile, workgroups */
 int streamk_amd_plan(int m, int n, int k, int cus, int* out);
+
+/* out[0], out[1] = row and column tile of tile number `tile` (0 <= tile <
+ * tiles_m * tiles_n); for tests of the numbering */
+void streamk_amd_tile_coord(int tile, int tiles_m, int tiles_n, int* out);
 
 /* text of the last STREAMK_ERR_RUNTIME on this thread */
 const char* streamk_amd_last_error(void);
