@@ -240,9 +240,7 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
         if (h == 1) {
           __builtin_amdgcn_s_waitcnt(0);  // my loads of the next slab and my reads of this one
           __builtin_amdgcn_s_barrier();
-#ifndef DN_SKIP_LOADS
           issue_slab(s + 2, (int)(cur != 0));
-#endif
         }
         dn_read16<0>(bn, w[h ^ 1][0]);
         dn_read16<2048>(bn, w[h ^ 1][1]);
