@@ -256,6 +256,15 @@ def main():
                                 "note": "cache-warm kernel time on other hardware, not comparable"}
         if main_name == "decode" else None,
     }
+    if args.shape == "headline":
+        # the sibling dense fp16 GEMM with its stream-K tail, on the reference's three
+        # examples (gemm/readme.md:29-31); its own program is gemm_streamk.py
+        import gemm_streamk
+        out["dense_streamk"] = [
+            {k: v for k, v in gemm_streamk.run(m, n, k, repeat=50, log=lambda *_: None).items()
+             if k in ("value", "unit", "ms_per_step", "config", "roofline", "vendor_library_tflops",
+                      "cos_similarity", "check")}
+            for (m, n, k) in [(4096, 4352, 4096), (4096, 4352, 10240), (1152, 4352, 4096)]]
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(O, main_name)
     print(json.dumps(out))
