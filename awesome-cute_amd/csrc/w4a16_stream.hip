@@ -365,9 +365,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     const int bl = ONE_TILE ? bf + p.wpt - 1 : tile_last_block(plan, t);
     bool writer = true;
     if (bl > bf) {
-      // a slot is two copies of MB*4*2*64 f4: [0] written back lazily by this
-      // XCD's L2, [1] written through to memory
-      constexpr int part_bytes = MB * 4 * 2 * 64 * 16;  // a slot: MB*4*2*64 f4
+      constexpr int part_bytes = MB * 4 * 2 * 64 * 16;  // a slot: MB*4*2*64 f4, written through
       const __amdgpu_buffer_rsrc_t rP = make_rsrc(p.scratch, 0x7fffffffu);
       // slot of work index b for this tile
       auto slot_of = [&](int b) { return ONE_TILE ? 2 * b : partial_slot(plan, b, t); };
