@@ -43,14 +43,22 @@ namespace w4a16 {
 
 namespace {
 
-constexpr int kDnTile = 256;     // rows and columns of a tile of C
+constexpr int kDnTile = 256;     // columns of a tile of C, and rows of the large tile
 constexpr int kDnStageK = 64;    // k depth of a stage (two MFMA k steps)
 constexpr int kDnRing = 2;       // slabs in LDS
-constexpr int kDnSlabA = 32 * 1024;
-constexpr int kDnSlab = 64 * 1024;
-constexpr int kDnLds = kDnRing * kDnSlab;
 constexpr int kDnOob = (int)0x80000000;
-constexpr int kDnPartBytes = kDnTile * kDnTile * 4;  // fp32 partial sums of one slice
+constexpr int kDnPartBytes = kDnTile * kDnTile * 4;  // fp32 partial sums of one slice (large tile)
+
+// LDS geometry for tiles of TM rows (256, or 128 when the large tiles are too
+// few for the compute units): a slab is TM rows of A and 256 rows of B
+template <int TM>
+struct DnShape {
+  static constexpr int kSlabA = TM * 128;
+  static constexpr int kSlab = kSlabA + kDnTile * 128;
+  static constexpr int kLds = kDnRing * kSlab;
+  static constexpr int kRB = TM / 32;                 // 16-row blocks per wave
+  static constexpr int kPartBytes = TM * kDnTile * 4;
+};
 constexpr int kDnMaxSlots = 256;                     // slices in flight per launch
 constexpr int kDnMaxSlices = 4;
 
@@ -59,6 +67,7 @@ struct DenseArgs {
   const void* B;
   void* C;
   int M, N, K;
+  int tile_rows;  // 256 or 128
   int tiles_m, tiles_n;
   int dp_tiles;  // tiles computed by one workgroup each
   int sk_tiles;  // tiles (the last ones in tile order) cut into ksplit slices
@@ -119,15 +128,21 @@ constexpr int dn_vmcnt(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 
 
 }  // namespace
 
+template <int TM>
 __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];  // kDnLds
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // DnShape<TM>::kLds
+  constexpr int RB = DnShape<TM>::kRB;
+  constexpr int kDnSlabA = DnShape<TM>::kSlabA;
+  constexpr int kDnSlab = DnShape<TM>::kSlab;
+  constexpr int kDnLds = DnShape<TM>::kLds;
+  constexpr int kPart = DnShape<TM>::kPartBytes;
   __shared__ int s_ticket;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int kg = lane >> 4;
   const int nu = lane & 15;
-  const int wm = wave >> 2;  // 128-row half of the tile
+  const int wm = wave >> 2;  // row half of the tile
   const int wn = wave & 3;   // 64-column quarter
 
   // stream-K slices come first in the grid, so that they run beside the first
@@ -149,28 +164,30 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   }
   int tm, tn;
   dn_tile_coord(tile, p.tiles_m, p.tiles_n, &tm, &tn);
-  const int m0 = tm * kDnTile;
+  const int m0 = tm * TM;
   const int n0 = tn * kDnTile;
-  const int rows = min(kDnTile, p.M - m0);
+  const int rows = min(TM, p.M - m0);
 
   const __amdgpu_buffer_rsrc_t rA =
       dn_rsrc((const char*)p.A + (size_t)m0 * p.K * 2, (unsigned)rows * (unsigned)p.K * 2u);
   const __amdgpu_buffer_rsrc_t rB =
       dn_rsrc((const char*)p.B + (size_t)n0 * p.K * 2, (unsigned)kDnTile * (unsigned)p.K * 2u);
 
-  // wave w fetches rows 32w ... 32w+31 of the A slab and of the B slab, eight
-  // rows per instruction: lane (r = lane/8, c = lane%8) lands at [r][c] and
-  // fetches chunk c ^ r of its row.  Rows past the end of A repeat the last
-  // row (never stored).
-  int a_src[4], b_src[4];
+  // wave w fetches rows (TM/8) w ... of the A slab and 32w ... 32w+31 of the
+  // B slab, eight rows per instruction: lane (r = lane/8, c = lane%8) lands at
+  // [r][c] and fetches chunk c ^ r of its row.  Rows past the end of A repeat
+  // the last row (never stored).
+  constexpr int TA = TM / 64;  // A instructions per wave and stage
+  int a_src[TA], b_src[4];
   {
     const int r8 = lane >> 3, c = (lane & 7) ^ r8;
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      const int r = 32 * wave + 8 * t + r8;
+    for (int t = 0; t < TA; t++) {
+      const int r = 8 * TA * wave + 8 * t + r8;
       a_src[t] = (r < rows ? r : rows - 1) * p.K * 2 + 16 * c;
-      b_src[t] = r * p.K * 2 + 16 * c;
     }
+#pragma unroll
+    for (int t = 0; t < 4; t++) b_src[t] = (32 * wave + 8 * t + r8) * p.K * 2 + 16 * c;
   }
   // this workgroup's stages [st0, st1) of the K/64 stages
   const int stages_all = p.K / kDnStageK;
@@ -181,17 +198,19 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   auto issue_slab = [&](int s, int ring) {
     const int inv = s < stages ? 0 : kDnOob;  // a stage past the end fetches zeros
     const int at = (st0 + s) * (kDnStageK * 2);
-    char* base = smem + ring * kDnSlab + (32 * wave) * 128;
+    char* base = smem + ring * kDnSlab;
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      dn_dma16(rA, base + t * 1024, a_src[t] | inv, at);
-      dn_dma16(rB, base + kDnSlabA + t * 1024, b_src[t] | inv, at);
-    }
+    for (int t = 0; t < TA; t++)
+      dn_dma16(rA, base + (8 * TA * wave + 8 * t) * 128, a_src[t] | inv, at);
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+      dn_dma16(rB, base + kDnSlabA + (32 * wave + 8 * t) * 128, b_src[t] | inv, at);
   };
+  constexpr int kSlabLoads = TA + 4;  // per wave
 
-  f4 acc[8][4];
+  f4 acc[RB][4];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < RB; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
@@ -202,14 +221,14 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
 #pragma unroll
   for (int h = 0; h < 2; h++) {
     const unsigned sw = 16 * ((4 * h + kg) ^ (nu & 7));
-    a_rd[h] = (unsigned)(size_t)smem + (128 * wm + nu) * 128 + sw;
+    a_rd[h] = (unsigned)(size_t)smem + (16 * RB * wm + nu) * 128 + sw;
     b_rd[h] = (unsigned)(size_t)smem + kDnSlabA + (64 * wn + nu) * 128 + sw;
   }
 
   // prologue: slabs 0 and 1 requested; slab 0 landed; its first operands read
   issue_slab(0, 0);
   issue_slab(1, 1);
-  __builtin_amdgcn_s_waitcnt(dn_vmcnt(8));
+  __builtin_amdgcn_s_waitcnt(dn_vmcnt(kSlabLoads));
   __builtin_amdgcn_s_barrier();
   dn_read16<0>(b_rd[0], w[0][0]);
   dn_read16<2048>(b_rd[0], w[0][1]);
@@ -220,23 +239,26 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   dn_read16<4096>(a_rd[0], af[2]);
 
   // One k step (H) of the stage in slab `cur`.  LDS reads in issue order, with
-  // Ai the operand of row block i and primes the prefetches for the step after:
+  // Ai the operand of row block i and primes the prefetches for the step after
+  // (eight row blocks per wave; with four the same three-ahead pattern):
   //   step 0:  | B(step 1) x4  A3 | A4 | A5 | A6 | A7 | A0' | A1' | A2' |
   //   step 1:  | A3 | A4 | A5 | A6 | A7 | barrier, B(next stage) x4  A0' | A1' | A2' |
   // When row block i is used, the reads issued after Ai may still be pending:
-  // three A operands, plus the four B reads where those were issued in between.
+  // three A operands, plus the four B reads where those were issued in between
+  // (the three row blocks from the one that issues them).
   // The barrier of a stage sits where the first read from the next slab is
   // about to be issued: by then every wave has its own part of that slab (it
   // waits for its loads first) and has issued and received all its reads of
   // the current slab, which the request for the stage after next overwrites.
   auto kstep = [&](auto H, unsigned cur, unsigned nxt, int s) {
     constexpr int h = decltype(H)::value;
+    constexpr int ib = h ? RB - 3 : 0;  // row block that issues the B reads
     const unsigned ac = a_rd[h] + cur;                        // this step, this slab
     const unsigned an = h ? a_rd[0] + nxt : a_rd[1] + cur;    // the step after
     const unsigned bn = h ? b_rd[0] + nxt : b_rd[1] + cur;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if ((h == 0 && i == 0) || (h == 1 && i == 5)) {
+    for (int i = 0; i < RB; i++) {
+      if (i == ib) {
         if (h == 1) {
           __builtin_amdgcn_s_waitcnt(0);  // my loads of the next slab and my reads of this one
           __builtin_amdgcn_s_barrier();
@@ -247,17 +269,25 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
         dn_read16<4096>(bn, w[h ^ 1][2]);
         dn_read16<6144>(bn, w[h ^ 1][3]);
       }
+      // operand of row block i + 3: of this step, or of the step after
+      auto frag = [&](auto I) {
+        constexpr int ii = decltype(I)::value;
+        if constexpr (ii < RB)
+          dn_read16<ii * 2048>(ac, af[ii & 3]);
+        else
+          dn_read16<(ii - RB) * 2048>(an, af[ii & 3]);
+      };
       switch (i) {  // i is a constant after unrolling
-        case 0: dn_read16<3 * 2048>(ac, af[3]); break;
-        case 1: dn_read16<4 * 2048>(ac, af[0]); break;
-        case 2: dn_read16<5 * 2048>(ac, af[1]); break;
-        case 3: dn_read16<6 * 2048>(ac, af[2]); break;
-        case 4: dn_read16<7 * 2048>(ac, af[3]); break;
-        case 5: dn_read16<0 * 2048>(an, af[0]); break;
-        case 6: dn_read16<1 * 2048>(an, af[1]); break;
-        case 7: dn_read16<2 * 2048>(an, af[2]); break;
+        case 0: frag(std::integral_constant<int, 3>{}); break;
+        case 1: frag(std::integral_constant<int, 4>{}); break;
+        case 2: frag(std::integral_constant<int, 5>{}); break;
+        case 3: frag(std::integral_constant<int, 6>{}); break;
+        case 4: frag(std::integral_constant<int, 7>{}); break;
+        case 5: frag(std::integral_constant<int, 8>{}); break;
+        case 6: frag(std::integral_constant<int, 9>{}); break;
+        case 7: frag(std::integral_constant<int, 10>{}); break;
       }
-      if ((h == 0 && i < 3) || (h == 1 && i >= 5))
+      if (i >= ib && i <= ib + 2)
         dn_wait<7>(af[i & 3]);
       else
         dn_wait<3>(af[i & 3]);
@@ -289,10 +319,10 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   // slices in slice order (its own from registers at its place in that order).
   if (ksplit > 1) {
     const __amdgpu_buffer_rsrc_t rP = dn_rsrc(p.scratch, 0x7fffffffu);
-    const int at = (wave * 32 * 64 + lane) * 16;
-    const int mine = work * kDnPartBytes;
+    const int at = (wave * (RB * 4) * 64 + lane) * 16;
+    const int mine = work * kPart;
 #pragma unroll
-    for (int i = 0; i < 8; i++)
+    for (int i = 0; i < RB; i++)
 #pragma unroll
       for (int j = 0; j < 4; j++)
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, acc[i][j]), rP,
@@ -308,11 +338,11 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     // one row block at a time: the other slices' values are requested
     // together, then added in slice order with my own at its place
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < RB; i++) {
       f4 v[kDnMaxSlices][4];
 #pragma unroll
       for (int k2 = 0; k2 < kDnMaxSlices; k2++) {
-        const int theirs = (sk_tile * ksplit + k2) * kDnPartBytes;
+        const int theirs = (sk_tile * ksplit + k2) * kPart;
         const int inv = (k2 < ksplit && k2 != ks) ? 0 : kDnOob;  // no traffic for the rest
 #pragma unroll
         for (int j = 0; j < 4; j++)
@@ -334,11 +364,12 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   }
 
   // ---- C: a lane holds, per (i, j), row 16i + nu and four consecutive
-  // columns.  The fp16 tile goes through LDS (the slabs are dead), one 128-row
-  // half at a time, and leaves as whole 512-byte rows with 16-byte stores;
+  // columns.  The fp16 tile goes through LDS (the slabs are dead), one half of
+  // its rows at a time, and leaves as whole 512-byte rows with 16-byte stores;
   // 8-byte stores straight from the registers cost 13 us more at 4096^3.
   constexpr int kPitch = kDnTile * 2 + 16;  // bytes per tile row in LDS
-  static_assert(128 * kPitch <= kDnLds, "");
+  constexpr int HR = TM / 2;                // rows of a half
+  static_assert(HR * kPitch <= kDnLds, "");
   half_t* C = (half_t*)p.C;
   const int q = lane >> 4;
 #pragma unroll
@@ -346,7 +377,7 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     __syncthreads();
     if (wm == hlf) {
 #pragma unroll
-      for (int i = 0; i < 8; i++)
+      for (int i = 0; i < RB; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
           const h4 o = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2],
@@ -356,10 +387,10 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     }
     __syncthreads();
 #pragma unroll
-    for (int it = 0; it < 8; it++) {
+    for (int it = 0; it < HR / 16; it++) {
       const int piece = it * 512 + tid;  // 16-byte piece of the half tile
       const int r = piece >> 5, c16 = piece & 31;
-      const int m = 128 * hlf + r;
+      const int m = HR * hlf + r;
       if (m < rows) {
         const i4 v = *(const i4*)(smem + r * kPitch + c16 * 16);
         *(i4*)(C + (size_t)(m0 + m) * p.N + n0 + c16 * 8) = v;
@@ -402,7 +433,7 @@ std::mutex g_dn_mu;
 DnDevice g_dn[kDnMaxDevices];
 
 struct DnPlan {
-  int tiles_m, tiles_n, dp_tiles, sk_tiles, ksplit, grid;
+  int tile_rows, tiles_m, tiles_n, dp_tiles, sk_tiles, ksplit, grid;
 };
 
 // Whole waves of tiles go to one workgroup each; the tiles of the partial last
@@ -411,7 +442,10 @@ struct DnPlan {
 // finishes a tile costs more than the slices save), each at least 256 deep.
 DnPlan dn_plan(int m, int n, int k, int cus) {
   DnPlan pl;
-  pl.tiles_m = ceil_div(m, kDnTile);
+  // 256 x 256 tiles, unless they would occupy at most half of the compute
+  // units: then 128 x 256 tiles, twice as many
+  pl.tile_rows = (2LL * ceil_div(m, kDnTile) * (n / kDnTile) <= cus) ? 128 : kDnTile;
+  pl.tiles_m = ceil_div(m, pl.tile_rows);
   pl.tiles_n = n / kDnTile;
   const int tiles = pl.tiles_m * pl.tiles_n;
   const int rem = cus > 0 ? tiles % cus : 0;
@@ -489,8 +523,11 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
       }
       cus = d.cus;
       if (!d.configured) {
-        e = hipFuncSetAttribute((const void*)dense_kernel,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kDnLds);
+        e = hipFuncSetAttribute((const void*)dense_kernel<256>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, DnShape<256>::kLds);
+        if (e == hipSuccess)
+          e = hipFuncSetAttribute((const void*)dense_kernel<128>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, DnShape<128>::kLds);
         if (e != hipSuccess) {
           dn_set_error(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
           break;
@@ -522,6 +559,7 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.M = m;
     a.N = n;
     a.K = k;
+    a.tile_rows = pl.tile_rows;
     a.tiles_m = pl.tiles_m;
     a.tiles_n = pl.tiles_n;
     a.dp_tiles = pl.dp_tiles;
@@ -529,7 +567,10 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.ksplit = pl.ksplit;
     a.locks = (int*)((char*)scratch + kDnPartialBytes);
     a.scratch = scratch;
-    hipLaunchKernelGGL(dense_kernel, dim3(pl.grid), dim3(512), kDnLds, stream, a);
+    if (pl.tile_rows == 128)
+      hipLaunchKernelGGL(dense_kernel<128>, dim3(pl.grid), dim3(512), DnShape<128>::kLds, stream, a);
+    else
+      hipLaunchKernelGGL(dense_kernel<256>, dim3(pl.grid), dim3(512), DnShape<256>::kLds, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) {
       dn_set_error(e, "kernel launch");
@@ -553,6 +594,7 @@ int streamk_amd_plan(int m, int n, int k, int cus, int* out) {
   out[3] = pl.sk_tiles;
   out[4] = pl.ksplit;
   out[5] = pl.grid;
+  out[6] = pl.tile_rows;
   return STREAMK_OK;
 }
 

@@ -35,9 +35,11 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
 int streamk_amd_check(int m, int n, int k);
 
 /* the tile split for a device with `cus` compute units (counterpart of
- * SK_DP_Block_Wrapper, dp_sk_block.h:31-80): out[0..5] = tiles along m, tiles
- * along n (256 x 256 tiles, numbered in panels of 8 column tiles), data-parallel tiles, stream-K
- * tiles (the last ones in tile order), k slices per stream-K tile, workgroups */
+ * SK_DP_Block_Wrapper, dp_sk_block.h:31-80): out[0..6] = tiles along m, tiles
+ * along n (tiles numbered in panels of 8 column tiles), data-parallel tiles, stream-K
+ * tiles (the last ones in tile order), k slices per stream-K tile, workgroups,
+ * rows of a tile (256, or 128 when 256 x 256 tiles would occupy at most half
+ * of the compute units; tiles are 256 columns wide) */
 int streamk_amd_plan(int m, int n, int k, int cus, int* out);
 
 /* out[0], out[1] = row and column tile of tile number `tile` (0 <= tile <

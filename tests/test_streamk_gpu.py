@@ -96,10 +96,11 @@ def test_one_hot_rows_return_rows_of_b(env):
     assert np.array_equal(C.view(np.uint16), B[:, np.arange(m) % k].T.copy().view(np.uint16))
 
 
-@pytest.mark.parametrize("m,n,k", [(4096, 4352, 4096), (1152, 4352, 4096), (4096, 4352, 10240)])
+@pytest.mark.parametrize("m,n,k", [(4096, 4352, 4096), (1152, 4352, 4096), (4096, 4352, 10240),
+                                   (4000, 4352, 512), (8100, 8192, 256)])
 def test_reference_examples(env, m, n, k):
-    """The reference's stream-K examples at full size (gemm/readme.md:27-31): a sample of
-    rows against the oracle, the whole result against torch's fp32 product by the
+    """The reference's stream-K examples at full size (gemm/readme.md:27-31), and two
+    shapes whose last row tile of 256 is partly empty: a sample of rows against the oracle, the whole result against torch's fp32 product by the
     reference's cosine criterion, and bit-identical results on a second run."""
     torch, streamk = env
     dev = torch.device("cuda:0")

@@ -54,7 +54,10 @@ def test_tile_split_properties(streamk, cus):
     for m, n, k in cases:
         rc, p = streamk.plan(m, n, k, cus)
         assert rc == 0
-        tiles = -(-m // 256) * (n // 256)
+        # 256 x 256 tiles, or 128 x 256 when the large ones would fill at most half the CUs
+        large = -(-m // 256) * (n // 256)
+        assert p["tile_rows"] == (128 if 2 * large <= cus else 256)
+        tiles = -(-m // p["tile_rows"]) * (n // 256)
         assert p["tiles_m"] * p["tiles_n"] == tiles
         assert p["dp_tiles"] + p["sk_tiles"] == tiles
         assert p["grid"] == p["dp_tiles"] + p["sk_tiles"] * p["k_slices"]
@@ -75,12 +78,16 @@ def test_tile_split_properties(streamk, cus):
 
 def test_reference_shapes_use_the_stream_k_tail(streamk):
     """The reference's stream-K examples (gemm/readme.md:27-31) have tile counts that
-    do not fill the compute units; all three get a stream-K part on 256 CUs."""
-    for m, n, k in [(4096, 4352, 4096), (4096, 4352, 10240), (1152, 4352, 4096)]:
+    do not fill the compute units.  On 256 CUs the two with 272 large tiles get a
+    stream-K part; the third has so few large tiles that it runs on 128-row tiles."""
+    for m, n, k in [(4096, 4352, 4096), (4096, 4352, 10240)]:
         rc, p = streamk.plan(m, n, k, 256)
-        assert rc == 0 and p["sk_tiles"] > 0 and p["k_slices"] >= 2, (m, n, k, p)
+        assert rc == 0 and p["tile_rows"] == 256
+        assert p["dp_tiles"] == 256 and p["sk_tiles"] == 16 and p["k_slices"] == 4, (m, n, k, p)
+    rc, p = streamk.plan(1152, 4352, 4096, 256)
+    assert rc == 0 and p["tile_rows"] == 128 and p["dp_tiles"] + p["sk_tiles"] == 9 * 17
     rc, p = streamk.plan(4096, 4096, 4096, 256)
-    assert p["sk_tiles"] == 0 and p["dp_tiles"] == 256
+    assert p["sk_tiles"] == 0 and p["dp_tiles"] == 256 and p["tile_rows"] == 256
 
 
 @pytest.mark.parametrize("tm,tn", [(16, 17), (5, 17), (1, 1), (3, 8), (7, 9), (32, 32), (2, 40)])
