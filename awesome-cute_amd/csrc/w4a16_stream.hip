@@ -76,8 +76,10 @@ struct StreamLds {
   // memory, which leaves room for a deeper ring.
   static constexpr bool kAliased = ONE_TILE && kDmaA;
   static constexpr int kRingBase = kAliased ? 0 : kReduceBytes;
+  // ... and all row blocks are reduced in one pass (kReduceBytes each)
   static constexpr int kBytes =
-      kAliased ? (4 * kRingBytesPerWave > kReduceBytes ? 4 * kRingBytesPerWave : kReduceBytes)
+      kAliased ? (4 * kRingBytesPerWave > MB * kReduceBytes ? 4 * kRingBytesPerWave
+                                                            : MB * kReduceBytes)
                : kReduceBytes + 4 * kRingBytesPerWave;
 };
 
@@ -336,20 +338,42 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     if constexpr (Lds::kAliased) __builtin_amdgcn_s_waitcnt(kWaitVm0);
     lds_barrier();
     W4A16_STAMP(4)
+    if constexpr (Lds::kAliased) {
+      // room for all row blocks at once: two barriers instead of two per block
 #pragma unroll
-    for (int i = 0; i < MB; i++) {
-      f4* red = (f4*)smem;
+      for (int i = 0; i < MB; i++) {
+        f4* red = (f4*)smem + i * (Lds::kReduceBytes / 16);
 #pragma unroll
-      for (int j = 0; j < 8; j++) red[(wave * 8 + j) * 64 + lane] = acc[i][j];
-      lds_barrier();
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        f4 v = red[(0 * 8 + 2 * wave + h) * 64 + lane];
-#pragma unroll
-        for (int w = 1; w < 4; w++) v += red[(w * 8 + 2 * wave + h) * 64 + lane];
-        res[i][h] = v;
+        for (int j = 0; j < 8; j++) red[(wave * 8 + j) * 64 + lane] = acc[i][j];
       }
       lds_barrier();
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        const f4* red = (const f4*)smem + i * (Lds::kReduceBytes / 16);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          f4 v = red[(0 * 8 + 2 * wave + h) * 64 + lane];
+#pragma unroll
+          for (int w = 1; w < 4; w++) v += red[(w * 8 + 2 * wave + h) * 64 + lane];
+          res[i][h] = v;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        f4* red = (f4*)smem;
+#pragma unroll
+        for (int j = 0; j < 8; j++) red[(wave * 8 + j) * 64 + lane] = acc[i][j];
+        lds_barrier();
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          f4 v = red[(0 * 8 + 2 * wave + h) * 64 + lane];
+#pragma unroll
+          for (int w = 1; w < 4; w++) v += red[(w * 8 + 2 * wave + h) * 64 + lane];
+          res[i][h] = v;
+        }
+        lds_barrier();
+      }
     }
 
     W4A16_STAMP(5)
