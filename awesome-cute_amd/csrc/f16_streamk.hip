@@ -399,6 +399,13 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   }
 }
 
+// C = 0 for an empty k range (a kernel rather than a memset, so that the call
+// can be captured into a HIP graph like any other)
+__global__ void dense_zero_kernel(half_t* C, size_t count) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) C[i] = (half_t)0.f;
+}
+
 }  // namespace w4a16
 
 // ---------------------------------------------------------------------------
@@ -480,9 +487,12 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
   int rc = dn_check(m, n, k);
   if (rc != STREAMK_OK || m == 0 || n == 0) return rc;
   if (k == 0) {  // an empty sum
-    hipError_t e = hipMemsetAsync(C, 0, (size_t)m * n * 2, stream);
+    const size_t count = (size_t)m * n;
+    hipLaunchKernelGGL(dense_zero_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0,
+                       stream, (half_t*)C, count);
+    hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
-      dn_set_error(e, "hipMemsetAsync");
+      dn_set_error(e, "kernel launch");
       return STREAMK_ERR_RUNTIME;
     }
     return STREAMK_OK;
