@@ -157,3 +157,32 @@ def test_degenerate_sizes_and_errors(env):
     with pytest.raises(ValueError):
         streamk.gemm(torch.zeros((16, 64), dtype=torch.half, device=dev),
                      torch.zeros((256, 128), dtype=torch.half, device=dev))
+
+
+def test_graph_replays_match_eager(env):
+    """A captured stream-K launch replayed several times, with eager launches and
+    synchronisations in between, gives the eager result every time (the tile counters
+    are handed back zeroed by the kernel itself, nothing in the launch is a memset)."""
+    torch, streamk = env
+    dev = torch.device("cuda:0")
+    A, B = inputs(700, 768, 1024, 5)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev)
+    A2, B2 = inputs(256, 512, 2048, 6)
+    dA2, dB2 = torch.from_numpy(A2).to(dev), torch.from_numpy(B2).to(dev)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        want = streamk.gemm(dA, dB).clone()      # also allocates this stream's scratch
+        other = streamk.gemm(dA2, dB2).clone()
+        side.synchronize()
+        C = torch.zeros_like(want)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            streamk.gemm(dA, dB, C)
+    for _ in range(4):
+        C.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(C, want)
+        with torch.cuda.stream(side):
+            assert torch.equal(streamk.gemm(dA2, dB2), other)
+            side.synchronize()
