@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/w4a16_known_answers.npz.
+"""Writes tests/golden/w4a16_known_answers.npz and tests/golden/f16_gemm_known_answers.npz.
 
 The reference keeps no golden vectors for this path, and nothing of it was
 imported or run to make these: they are known answers produced by this
@@ -9,7 +9,8 @@ packers or the kernels that alters any bit shows up as a diff against data
 instead of passing silently.  Two small problems (group 128 and per-channel
 scales): logical int4 weights and scales, their packed forms, activations, the
 dequantised weight matrix, the fp32-accumulate GEMM result, and the three
-layout permutations.
+layout permutations.  For the dense fp16 GEMM (whose reference program keeps
+no vectors either): two small problems with their fp32-accumulate results.
 
 Run from the repository root:  python tests/golden/make_fixtures.py
 """
@@ -47,6 +48,17 @@ def main():
     out["perm"], out["scale_perm"], out["scale_perm_single"] = perm, sp, sps
     path = os.path.join(HERE, "w4a16_known_answers.npz")
     np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes")
+
+    dense = {}
+    for tag, (M, N, K, seed) in {"a": (40, 256, 192, 21), "b": (130, 256, 320, 22)}.items():
+        rng = np.random.default_rng(seed)
+        A = (rng.random((M, K)) * 4 - 2).astype(np.float16)
+        B = (rng.random((N, K)) * 4 - 2).astype(np.float16)
+        dense[f"{tag}_A"], dense[f"{tag}_B"] = A.view(np.uint16), B.view(np.uint16)
+        dense[f"{tag}_C"] = O.dense_gemm_tn(A, B).view(np.uint16)
+    path = os.path.join(HERE, "f16_gemm_known_answers.npz")
+    np.savez_compressed(path, **dense)
     print(path, os.path.getsize(path), "bytes")
 
 

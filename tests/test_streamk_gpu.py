@@ -186,3 +186,11 @@ def test_graph_replays_match_eager(env):
         with torch.cuda.stream(side):
             assert torch.equal(streamk.gemm(dA2, dB2), other)
             side.synchronize()
+
+
+@pytest.mark.parametrize("tag", ["a", "b"])
+def test_frozen_known_answers(env, tag):
+    """The committed known answers (tests/golden/f16_gemm_known_answers.npz)."""
+    z = np.load(os.path.join(ROOT, "tests", "golden", "f16_gemm_known_answers.npz"))
+    A, B = z[f"{tag}_A"].view(np.float16), z[f"{tag}_B"].view(np.float16)
+    close(gpu_gemm(env, A, B), z[f"{tag}_C"].view(np.float16))

@@ -130,3 +130,12 @@ def test_gemm_refuses_cpu_tensors(streamk):
     import torch
     with pytest.raises(ValueError):
         streamk.gemm(torch.zeros((16, 64), dtype=torch.half), torch.zeros((256, 64), dtype=torch.half))
+
+
+def test_dense_oracle_reproduces_frozen_known_answers():
+    """tests/golden/f16_gemm_known_answers.npz (this repository's own known answers, the
+    reference program keeps none): the oracle still gives every bit of them."""
+    z = np.load(os.path.join(ROOT, "tests", "golden", "f16_gemm_known_answers.npz"))
+    for tag in ("a", "b"):
+        A, B = z[f"{tag}_A"].view(np.float16), z[f"{tag}_B"].view(np.float16)
+        assert np.array_equal(O.dense_gemm_tn(A, B).view(np.uint16), z[f"{tag}_C"])
