@@ -7,8 +7,9 @@
 // range (the slices meet through the same ticketed exchange as the streaming
 // kernel's).  Waves 0-3 run the first half of the workgroup's k range and
 // waves 4-7 the second half over the same tile, and the two halves are added
-// through LDS at the end.  Two waves per SIMD matter: a wave cannot issue its own unpack/LDS
-// instructions under its own MFMAs, but the other wave's run there for free.
+// through LDS at the end.  Two waves per SIMD matter: a wave pays 11 to 22
+// cycles of its own issue time for every LDS or global instruction, and the
+// other wave's MFMAs run there.
 // Within a half, wave w keeps a 16*RB x 64 fp32 accumulator (16*RB registers):
 // columns 16j+8h+c of the two 64-column blocks 2p, 2p+1 with p = w/2 and
 // j in {2(w%2), 2(w%2)+1}.
@@ -22,8 +23,8 @@
 //     stored in the k-slot order the weight layout dictates so that an
 //     operand is one conflict-free ds_read_b128.
 // Per 32-deep k step a wave issues 32 MFMAs, 8 LDS reads and the unpack of 4
-// weight words (about 52 VALU instructions), software-pipelined one step
-// ahead.
+// weight words (52 VALU instructions), software-pipelined one step ahead and
+// dealt out two behind every MFMA, where they cost no issue time.
 #include "w4a16_common.hpp"
 
 // Tuning builds may remap the k stage that is fetched (e.g. to a cache-hot
@@ -236,11 +237,51 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     af[idx] = *(const i4*)(step_base + a_rd + i * 256);
   };
 
+  // One operation of the unpack of word bw[r][j2] into w[buf] (the sequence of
+  // dequant_word, cut up so that it can be dealt out between the MFMAs):
+  // op 0 the shift, 1-4 the four mask-and-exponent words, 5-8 the bias
+  // removal, 9-12 (group mode) the scale.
+  int wt[2];  // the shifted words
+  auto dq_op = [&](int buf, int slot, int j2, int r, int op) {
+    const h2 sub = {(half_t)1032.f, (half_t)1032.f};
+    const h2 mul = {(half_t)0.0625f, (half_t)0.0625f};
+    const h2 add = {(half_t)-72.f, (half_t)-72.f};
+    i4& lo = *(i4*)&w[buf][2 * j2];      // column c: dwords 2r (k pair 2t), 2r+1 (k pair 2t+8)
+    i4& hi = *(i4*)&w[buf][2 * j2 + 1];  // column c+8
+    const int q = bw[r][j2];
+    switch (op) {
+      case 0: wt[r] = (int)((unsigned)q >> 8); break;
+      case 1: lo[2 * r] = (q & dc.lo_mask) | dc.ex; break;
+      case 2: lo[2 * r + 1] = (q & dc.hi_mask) | dc.ex; break;
+      case 3: hi[2 * r] = (wt[r] & dc.lo_mask) | dc.ex; break;
+      case 4: hi[2 * r + 1] = (wt[r] & dc.hi_mask) | dc.ex; break;
+      case 5: lo[2 * r] = as_int(as_h2(lo[2 * r]) - sub); break;
+      case 6: lo[2 * r + 1] = as_int(__builtin_elementwise_fma(as_h2(lo[2 * r + 1]), mul, add)); break;
+      case 7: hi[2 * r] = as_int(as_h2(hi[2 * r]) - sub); break;
+      case 8: hi[2 * r + 1] = as_int(__builtin_elementwise_fma(as_h2(hi[2 * r + 1]), mul, add)); break;
+      default: {
+        const h2 s2 = as_h2(sreg[slot][j2]);
+        const h2 s0 = {s2[0], s2[0]};
+        const h2 s1 = {s2[1], s2[1]};
+        if (op == 9) lo[2 * r] = as_int(as_h2(lo[2 * r]) * s0);
+        if (op == 10) lo[2 * r + 1] = as_int(as_h2(lo[2 * r + 1]) * s0);
+        if (op == 11) hi[2 * r] = as_int(as_h2(hi[2 * r]) * s1);
+        if (op == 12) hi[2 * r + 1] = as_int(as_h2(hi[2 * r + 1]) * s1);
+      }
+    }
+  };
+
   // One 32-deep k step: 4*RB MFMAs on w[h] and the operand ring, while the
   // operands of the next step are fetched from LDS and its weights unpacked
-  // into w[h^1].  `mid` runs half way through the row blocks.
+  // into w[h^1].  Two VALU instructions issued behind an MFMA cost nothing, a
+  // third costs its full four cycles, so the unpack is dealt out two (with 64
+  // rows: four) operations per MFMA instead of standing in blocks between
+  // them; scheduling fences keep it that way.  `extra(m)` runs behind MFMA m.
   auto step = [&](int h, const char* cur_base, const char* nxt_base, const char* nxt_stage,
-                  int nslot, int nh, auto&& mid) {
+                  int nslot, int nh, auto&& extra) {
+    constexpr int kOpsPerWord = GROUP ? 13 : 9;
+    constexpr int kPairsPerMfma = RB == 8 ? 1 : 2;  // one operation of each word of a pair
+    constexpr int kFirst = RB == 8 ? 6 : 3;         // the words are read from LDS behind MFMA 0
 #pragma unroll
     for (int i = 0; i < RB; i++) {
       if (i == 0) read_bw(nxt_stage, nh);
@@ -250,11 +291,52 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
         read_frag((i + 3) & 3, nxt_base, i + 3 - RB);
       const h8 a = __builtin_bit_cast(h8, af[i & 3]);
 #pragma unroll
-      for (int j = 0; j < 4; j++)
+      for (int j = 0; j < 4; j++) {
+        const int m = 4 * i + j;
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[h][j], a, acc[i][j], 0, 0, 0);
-      if (i == RB / 4) dequant_pair(h ^ 1, nslot, nh, 0);
-      if (i == RB / 2 - 1) mid();
-      if (i == RB / 2 + RB / 8) dequant_pair(h ^ 1, nslot, nh, 1);
+#pragma unroll
+        for (int u = 0; u < kPairsPerMfma; u++) {
+          const int t = (m - kFirst) * kPairsPerMfma + u;
+#ifndef W4A16_PF_SKIP_DQ
+          if (t >= 0 && t < 2 * kOpsPerWord) {
+            dq_op(h ^ 1, nslot, t / kOpsPerWord, 0, t % kOpsPerWord);
+            dq_op(h ^ 1, nslot, t / kOpsPerWord, 1, t % kOpsPerWord);
+          }
+#endif
+        }
+        extra(m);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+
+  // The slab traffic of a stage, dealt out behind the MFMAs of its first step:
+  // each staging register is written to LDS (slab cs+1) and then requested
+  // again (slab cs+2), so every load has a whole stage to arrive.
+  auto stage_traffic = [&](int m, int ring_next, int s_next2) {
+    constexpr int kPerA = 5;  // four dword writes and the reload of one register
+    constexpr int kBegin = 4 * RB - (HB * kPerA + 2 * 2);
+    const int x = m - kBegin;
+    if (x < 0) return;
+#ifdef W4A16_PF_SKIP_TRAFFIC
+    return;
+#endif
+    char* base = smem + ring_next * kPfStageBytes;
+    const int sg = s_begin + s_next2;
+    const int inv = sg < s_end ? 0 : kOobPf;
+    if (x < HB * kPerA) {
+      const int i = x / kPerA, g = x % kPerA;
+      if (g < 4)
+        *(int*)(base + a_wr + g * kPlane + i * 32 * 16) = areg[i][g];
+      else
+        areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
+    } else {
+      const int y = x - HB * kPerA, i = y >> 1;
+      if ((y & 1) == 0)
+        *(i4*)(base + b_wr + i * 4096) = bcopy[i];
+      else
+        bcopy[i] = __builtin_amdgcn_raw_buffer_load_b128(
+            rB, b_ld | inv, (4 * W4A16_PF_K(sg) + 2 * i + (wave >> 1)) * b_row, 0);
     }
   };
 
@@ -272,9 +354,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   read_frag(1, smem, 1);
   read_frag(2, smem, 2);
 
-  // The instruction arbiter favours the older waves (the first k half), which
-  // then idle at every barrier; a higher priority for the second half evens
-  // the two out (measured: 4 % faster).
+  // The instruction arbiter favours the older waves (the first k half); a
+  // higher priority for the second half evens the two out (measured: never
+  // slower, up to 4 % faster depending on the schedule of the loop).
   if (kh) __builtin_amdgcn_s_setprio(1);
   int ring = 0;  // LDS slab of the stage being computed
   W4A16_PF_TBEGIN
@@ -289,15 +371,15 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       // The slab written here was last read two stages ago, and every wave
       // has passed the previous barrier since, so one barrier per stage is
       // enough; it sits mid-stage, where no wave needs the new slab yet.
-      step(0, cur, cur + kPfStepBytes, cur, u, 1, [&]() {
-        store_a(ring_next);
-        issue_a(cs + 2);
-      });
+      step(0, cur, cur + kPfStepBytes, cur, u, 1,
+           [&](int m) { stage_traffic(m, ring_next, cs + 2); });
       W4A16_PF_T0
+#ifndef W4A16_PF_NO_BARRIER
       __syncthreads();
+#endif
       W4A16_PF_T1
       // step 1: the scales of this stage are spent, request those of stage cs+2
-      step(1, cur + kPfStepBytes, nxt, nxt, u ^ 1, 0, [&]() {});
+      step(1, cur + kPfStepBytes, nxt, nxt, u ^ 1, 0, [](int) {});
       issue_s(u, cs + 2);
       ring = ring_next;
     }
