@@ -10,6 +10,14 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # the tests load the in-tree library; build it only if there is none
+    if not os.path.exists(os.path.join(ROOT, "awesome-cute_amd", "libmarlin_amd.so")):
+        import importlib.util
+        spec = importlib.util.spec_from_file_location(
+            "_build_marlin_amd", os.path.join(ROOT, "awesome-cute_amd", "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build_library()
 
 
 def _have_gpu():
