@@ -149,6 +149,9 @@ std::atomic<int> g_force_kernel{0};
 // 11008, 28672 x 8192}): filling the CUs pays up to four slices; more slices
 // only add partial-sum traffic.
 std::atomic<int> g_force_k_slices{0};
+// 0 = choose by cost, 64 or 128 = rows of C per prefill workgroup; set by
+// marlin_amd_force_tile_rows (tests and tools)
+std::atomic<int> g_force_tile_rows{0};
 
 int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
   int most = k / 256;
@@ -166,21 +169,48 @@ int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
 // Either kernel can do any problem whose n is a multiple of 256: the prefill
 // kernel once, or the streaming kernel once per 64 rows, reading the weights
 // again every time.  Costs in us, fitted to measurements on MI355X.
-double prefill_cost(int m, int n, int k, int cus) {
-  const int tile_rows = prefill_tile_rows(m);
+//
+// Prefill: a full-depth tile takes 6 + 0.0130 k with 128 rows and 5 + 0.0080 k
+// with 64 (every unpacked weight then meets four row blocks instead of eight,
+// so a 64-row tile costs more than half of a 128-row one) when the launch
+// fills the CUs; k slices divide that and add their exchange, 3 + 2 s (128
+// rows: 128 KiB of partial sums per workgroup) or 3 + 1.5 s (64 rows).
+double prefill_cost_rows(int m, int n, int k, int cus, int tile_rows) {
   const int tiles = ceil_div(m, tile_rows) * (n / 256);
   const int s = prefill_k_slices(tiles, tile_rows, k, cus);
-  const double rounds = ceil_div(tiles * s, cus);
-  // a full-depth tile takes 6 + 0.0108 k (two thirds of that with 64 rows)
-  // however few tiles there are; slices divide it and add their exchange
-  const double tile = (6.0 + 0.0108 * k) * (tile_rows == 64 ? 0.66 : 1.0);
-  return rounds * (tile / s + (s > 1 ? 5.0 + 2.5 * s : 0.0));
+  // more workgroups than CUs run in rounds, the last of which is faster the
+  // emptier it is: half way between whole rounds and the plain ratio fits
+  // (N = K = 4096, M = 3072: 384 tiles of 128 rows, 102.7 us, where one round
+  // of 256 takes 59.3)
+  const double ratio = (double)tiles * s / cus;
+  const double rounds = ratio <= 1.0 ? 1.0 : 0.5 * (ceil_div(tiles * s, cus) + ratio);
+  // ... and a launch that leaves CUs idle runs its tiles faster (clock, and
+  // fewer workgroups at the memory): 0.9 of the time at three quarters full
+  const double fill = ratio < 1.0 ? 0.6 + 0.4 * ratio : 1.0;
+  const double tile = (tile_rows == 64 ? 5.0 + 0.0080 * k : 6.0 + 0.0130 * k) * fill;
+  const double exchange = s > 1 ? 3.0 + (tile_rows == 64 ? 1.5 : 2.0) * s : 0.0;
+  return rounds * (tile / s + exchange);
+}
+
+// Rows of C per prefill workgroup.  64-row tiles are twice as many, so they
+// need fewer k slices to fill the CUs (or none), which wins while the problem
+// is small: at N = K = 4096 up to about 512 rows (M = 128: 16.0 against
+// 21.9 us), at N = 4096, K = 11008 up to 256 (27.5 against 38.9 us at M = 128).
+int prefill_tile_rows(int m, int n, int k, int cus) {
+  const int force = g_force_tile_rows.load(std::memory_order_relaxed);
+  if (force == 64 || force == 128) return force;
+  if (m <= 64) return 64;
+  return prefill_cost_rows(m, n, k, cus, 64) < prefill_cost_rows(m, n, k, cus, 128) ? 64 : 128;
+}
+
+double prefill_cost(int m, int n, int k, int cus) {
+  return prefill_cost_rows(m, n, k, cus, prefill_tile_rows(m, n, k, cus));
 }
 
 double stream_cost(int m, int n, int k) {
   const double mb = 0.5e-6 * n * k;  // MB of packed weights, read once per pass
   // a pass over 49-64 rows (4 row blocks); the slope flattens for big problems
-  const double full = mb <= 22.5 ? 11.6 + 0.52 * mb : 23.3 + 0.25 * (mb - 22.5);
+  const double full = mb <= 22.5 ? 9.8 + 0.60 * mb : 23.3 + 0.25 * (mb - 22.5);
   const int tail = m % kStreamMaxRows;
   double t = (m / kStreamMaxRows) * full;
   if (tail > 16)
@@ -208,7 +238,7 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
-    pl.tile_rows = prefill_tile_rows(m);
+    pl.tile_rows = prefill_tile_rows(m, n, k, cus);
     const int tiles = ceil_div(m, pl.tile_rows) * (n / 256);
     pl.ksplit = prefill_k_slices(tiles, pl.tile_rows, k, cus);
     pl.grid = tiles * pl.ksplit;
@@ -316,7 +346,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
       a.scratch = scratch;
       a.gpb = 0;
       a.wpt = 0;
-      rc = launch_prefill(a, groupsize != -1, pl.ksplit, stream);
+      rc = launch_prefill(a, groupsize != -1, pl.ksplit, pl.tile_rows, stream);
       if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
     } else if (pl.kernel == 1 && scratch) {
       rc = MARLIN_OK;
@@ -426,6 +456,10 @@ void marlin_amd_force_kernel(int which) {
 
 void marlin_amd_force_k_slices(int slices) {
   g_force_k_slices.store(slices > 0 ? slices : 0, std::memory_order_relaxed);
+}
+
+void marlin_amd_force_tile_rows(int rows) {
+  g_force_tile_rows.store(rows == 64 || rows == 128 ? rows : 0, std::memory_order_relaxed);
 }
 
 void marlin_amd_work_order(int grid, int* out) {

@@ -178,7 +178,7 @@ int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 // ksplit >= 1 slices of the k range per tile; above 1 the launch needs
 // a.scratch (ksplit * tiles * tile bytes of fp32) and a.locks (one zeroed
 // counter per tile, zero again afterwards)
-int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
-int prefill_tile_rows(int m);  // rows of C per prefill workgroup: 64 up to 64 rows, else 128
+// tile_rows: rows of C per workgroup, 64 or 128
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream);
 
 }  // namespace w4a16

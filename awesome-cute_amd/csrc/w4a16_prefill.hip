@@ -2,7 +2,7 @@
 // design minimises everything that competes with the matrix pipe.
 //
 // One workgroup of 8 waves (two per SIMD) owns a 16*RB-row x 256-column tile
-// of C (RB = 8 row blocks, or 4 when there are at most 64 rows) and, when the
+// of C (RB = 8 row blocks, or 4: the host's choice) and, when the
 // tiles alone would leave compute units idle, one of `ksplit` slices of the k
 // range (the slices meet through the same ticketed exchange as the streaming
 // kernel's).  Waves 0-3 run the first half of the workgroup's k range and
@@ -526,10 +526,8 @@ static void launch_rb(const GemmArgs& a, int ksplit, hipStream_t stream) {
                      stream, a, tiles_m, tiles_n, ksplit);
 }
 
-int prefill_tile_rows(int m) { return m <= 64 ? 64 : 128; }
-
-int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream) {
-  if (prefill_tile_rows(a.M) == 64) {
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream) {
+  if (tile_rows == 64) {
     if (group) launch_rb<true, 4>(a, ksplit, stream); else launch_rb<false, 4>(a, ksplit, stream);
   } else {
     if (group) launch_rb<true, 8>(a, ksplit, stream); else launch_rb<false, 8>(a, ksplit, stream);

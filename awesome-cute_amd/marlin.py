@@ -33,6 +33,8 @@ _lib.marlin_amd_plan.restype = _I
 _lib.marlin_amd_plan.argtypes = [_I] * 8 + [_P]
 _lib.marlin_amd_force_k_slices.restype = None
 _lib.marlin_amd_force_k_slices.argtypes = [_I]
+_lib.marlin_amd_force_tile_rows.restype = None
+_lib.marlin_amd_force_tile_rows.argtypes = [_I]
 _lib.marlin_amd_force_kernel.restype = None
 _lib.marlin_amd_force_kernel.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
@@ -238,6 +240,11 @@ def force_kernel(which):
 def force_k_slices(slices):
     """Slices of the k range per prefill tile; 0 = choose by cost (process-wide)."""
     _lib.marlin_amd_force_k_slices(int(slices))
+
+
+def force_tile_rows(rows):
+    """Rows of C per prefill workgroup (64 or 128); 0 = choose by cost (process-wide)."""
+    _lib.marlin_amd_force_tile_rows(int(rows))
 
 
 def work_order(grid):

@@ -118,6 +118,12 @@ void marlin_amd_force_kernel(int which);
  */
 void marlin_amd_force_k_slices(int slices);
 
+/*
+ * Rows of C per workgroup of the prefill kernel, process-wide: 0 = choose by
+ * cost (default), 64 or 128.  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_tile_rows(int rows);
+
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *marlin_amd_last_error(void);
 

@@ -221,16 +221,19 @@ def test_either_kernel_above_64_rows(env, which, m):
 @pytest.mark.parametrize("slices", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("m", [1, 16, 40, 64, 65, 128, 200, 384])
 def test_prefill_kernel_k_slices(env, m, slices):
-    """The prefill kernel at every tile height (64 rows up to 64, else 128) and
-    with its k range cut into slices that meet through the ticketed exchange;
-    the same slicing gives the same bits every time."""
+    """The prefill kernel at both tile heights (64 and 128 rows; up to 64 rows
+    the planner only uses the first) and with its k range cut into slices that
+    meet through the ticketed exchange; the same slicing gives the same bits
+    every time."""
     torch, marlin = env
+    rows = 64 if m <= 64 or (m + slices) % 2 else 128
     marlin.force_kernel(2)
     marlin.force_k_slices(slices)
+    marlin.force_tile_rows(rows)
     try:
         rc, plan = marlin.plan(m, 512, 2048, 128)
         assert rc == 0 and plan["kernel"] == 2 and plan["k_slices"] == slices
-        assert plan["tile_rows"] == (64 if m <= 64 else 128)
+        assert plan["tile_rows"] == rows
         check(env, m, 512, 2048, 128, seed=m + slices)
         check(env, m, 256, 1024, -1, seed=m + slices + 3)  # at most 4 slices of 256
         A, q, s, B, sp = O.make_problem(m, 768, 1536, 128, seed=5)
@@ -240,6 +243,25 @@ def test_prefill_kernel_k_slices(env, m, slices):
     finally:
         marlin.force_kernel(0)
         marlin.force_k_slices(0)
+        marlin.force_tile_rows(0)
+
+
+@pytest.mark.parametrize("rows", [64, 128])
+@pytest.mark.parametrize("m,n,k,g", [(130, 1024, 1024, 128), (300, 512, 2304, -1), (1000, 768, 512, 128),
+                                     (33, 512, 1024, 128)])
+def test_prefill_kernel_tile_rows(env, rows, m, n, k, g):
+    """Both tile heights on ragged row counts, several row tiles per column."""
+    torch, marlin = env
+    marlin.force_kernel(2)
+    marlin.force_tile_rows(rows)
+    try:
+        rc, plan = marlin.plan(m, n, k, g)
+        assert rc == 0 and plan["kernel"] == 2 and plan["tile_rows"] == rows
+        assert plan["grid"] == -(-m // rows) * (n // 256) * plan["k_slices"]
+        check(env, m, n, k, g, seed=m + rows)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_tile_rows(0)
 
 
 @pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol(marlin):
     names = re.findall(r"\b(marlin_\w+)\s*\(", header)
     assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
             "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_force_kernel",
-            "marlin_amd_force_k_slices",
+            "marlin_amd_force_k_slices", "marlin_amd_force_tile_rows",
             "marlin_amd_last_error",
             "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
@@ -191,13 +191,15 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
 def test_kernel_choice_by_cost(marlin):
     """Few rows go through the streaming kernel, many through the prefill
     kernel, whose k range is cut into up to four slices while tiles alone would
-    leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles.  The
-    knobs override the choice."""
+    leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
+    so do more rows while twice as many tiles save k slices.  The knobs override
+    the choice."""
     for m, n, k, kernel, slices, rows in [
             (1, 4096, 4096, 1, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
-            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (128, 4096, 4096, 2, 4, 128),
-            (512, 4096, 4096, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
-            (2048, 4096, 4096, 2, 1, 128)]:
+            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 2, 4, 64),
+            (128, 4096, 4096, 2, 4, 64), (512, 4096, 4096, 2, 2, 64),
+            (512, 4096, 11008, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
+            (1536, 4096, 4096, 2, 1, 128), (2048, 4096, 4096, 2, 1, 128)]:
         rc, p = marlin.plan(m, n, k, 128)
         assert rc == 0 and (p["kernel"], p["k_slices"], p["tile_rows"]) == (kernel, slices, rows), \
             (m, n, k, p)
@@ -209,7 +211,15 @@ def test_kernel_choice_by_cost(marlin):
         assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32
         marlin.force_kernel(2)
         rc, p = marlin.plan(100, 512, 1024, 128)
-        assert rc == 0 and p["kernel"] == 2 and p["grid"] == 2 * p["k_slices"]
+        assert rc == 0 and p["kernel"] == 2
+        assert p["grid"] == -(-100 // p["tile_rows"]) * 2 * p["k_slices"]
+        marlin.force_tile_rows(128)
+        assert marlin.plan(100, 512, 1024, 128)[1]["tile_rows"] == 128
+        assert marlin.plan(40, 512, 1024, 128)[1]["tile_rows"] == 128
+        marlin.force_tile_rows(64)
+        rc, p = marlin.plan(2048, 4096, 4096, 128)
+        assert rc == 0 and p["tile_rows"] == 64 and p["grid"] == 32 * 16 * p["k_slices"]
+        marlin.force_tile_rows(0)
         marlin.force_k_slices(3)
         assert marlin.plan(100, 512, 1024, 128)[1]["k_slices"] == 3
         assert marlin.plan(100, 512, 512, 128)[1]["k_slices"] == 2  # slices are >= 256 deep
@@ -217,6 +227,7 @@ def test_kernel_choice_by_cost(marlin):
     finally:
         marlin.force_kernel(0)
         marlin.force_k_slices(0)
+        marlin.force_tile_rows(0)
 
 
 def test_plan_picks_kernels(marlin):
