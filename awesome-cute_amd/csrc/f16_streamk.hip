@@ -191,8 +191,9 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   }
   // this workgroup's stages [st0, st1) of the K/64 stages
   const int stages_all = p.K / kDnStageK;
-  const int st0 = (int)((long long)ks * stages_all / ksplit);
-  const int st1 = (int)((long long)(ks + 1) * stages_all / ksplit);
+  // (at most 4 slices of at most 2^24 stages: 32 bits do)
+  const int st0 = (int)((unsigned)ks * (unsigned)stages_all / (unsigned)ksplit);
+  const int st1 = (int)((unsigned)(ks + 1) * (unsigned)stages_all / (unsigned)ksplit);
   const int stages = st1 - st0;
 
   auto issue_slab = [&](int s, int ring) {

@@ -79,6 +79,16 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   extern __shared__ __attribute__((aligned(16))) char smem_all[];  // PfShape<RB>::kLdsBytes
   __shared__ int s_ticket;
   W4A16_PF_TENTRY
+  {
+    // fetch every kernel argument in one round trip (the compiler would fetch
+    // the pointers in a second one, just before the first load needs them)
+    const void *a_ = p.A, *b_ = p.B, *s_ = p.S;
+    void* c_ = p.C;
+    int* l_ = p.locks;
+    float* sc_ = p.scratch;
+    asm volatile("" ::"s"(a_), "s"(b_), "s"(s_), "s"(c_), "s"(l_), "s"(sc_), "s"(p.M), "s"(p.N),
+                 "s"(p.K), "s"(tiles_m), "s"(tiles_n), "s"(ksplit));
+  }
   constexpr int kPfTileM = PfShape<RB>::kTileM;
   constexpr int kPlane = PfShape<RB>::kPlane;
   constexpr int kPfStepBytes = PfShape<RB>::kStepBytes;
@@ -147,8 +157,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // this half's stages: [s_begin, s_end) of the K/64 stages; the loop runs the
   // same count in both halves (a stage past s_end fetches zeros)
   const int stages_all = p.K / kPfStageK;
-  const int st0 = (int)((long long)ks * stages_all / ksplit);        // this workgroup's slice
-  const int st1 = (int)((long long)(ks + 1) * stages_all / ksplit);
+  // this workgroup's slice (at most 8 slices of at most 2^18 stages: 32 bits do)
+  const int st0 = (int)((unsigned)ks * (unsigned)stages_all / (unsigned)ksplit);
+  const int st1 = (int)((unsigned)(ks + 1) * (unsigned)stages_all / (unsigned)ksplit);
   const int half_stages = (st1 - st0 + 1) >> 1;
   const int s_begin = st0 + kh * half_stages;
   const int s_end = kh ? st1 : st0 + half_stages;
