@@ -107,16 +107,27 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   const int jp = wave & 1;   // pair of 16-column groups inside each block
 
   // Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a
-  // contiguous run of tiles (column tile fastest) so that the workgroups
-  // sharing an L2 read the same rows of A and neighbouring columns of B.
+  // contiguous run of tile numbers so that the workgroups sharing an L2 read
+  // the same rows of A and neighbouring columns of B.
   // The k slices of a tile are consecutive work indices, so they share an XCD.
   const int total = tiles_m * tiles_n * ksplit;
   int work = (int)blockIdx.x;
   if ((total & 7) == 0) work = (work & 7) * (total >> 3) + (work >> 3);
   const int tile = work / ksplit;
   const int ks = work - tile * ksplit;
-  const int tm = tile / tiles_n;
-  const int tn = tile - tm * tiles_n;
+  int tm, tn;
+  if ((tiles_n & 7) == 0) {
+    // tiles numbered in panels of 8 column tiles, row tile next: an XCD's run
+    // of tiles is then closer to square (4 x 8 instead of 2 x 16 at M = 2048,
+    // N = 4096) and shares more of A and B (8192 x 8192, M = 2048: 226 -> 221 us)
+    const int per_panel = 8 * tiles_m;
+    const int panel = tile / per_panel, within = tile - panel * per_panel;
+    tm = within >> 3;
+    tn = panel * 8 + (within & 7);
+  } else {
+    tm = tile / tiles_n;
+    tn = tile - tm * tiles_n;
+  }
   const int m0 = tm * kPfTileM;
   const int rows = min(kPfTileM, p.M - m0);
 

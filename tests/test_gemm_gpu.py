@@ -248,7 +248,7 @@ def test_prefill_kernel_k_slices(env, m, slices):
 
 @pytest.mark.parametrize("rows", [64, 128])
 @pytest.mark.parametrize("m,n,k,g", [(130, 1024, 1024, 128), (300, 512, 2304, -1), (1000, 768, 512, 128),
-                                     (33, 512, 1024, 128)])
+                                     (33, 512, 1024, 128), (300, 2048, 512, 128), (520, 4096, 256, -1)])
 def test_prefill_kernel_tile_rows(env, rows, m, n, k, g):
     """Both tile heights on ragged row counts, several row tiles per column."""
     torch, marlin = env
