@@ -394,7 +394,8 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
       const int m = HR * hlf + r;
       if (m < rows) {
         const i4 v = *(const i4*)(smem + r * kPitch + c16 * 16);
-        *(i4*)(C + (size_t)(m0 + m) * p.N + n0 + c16 * 8) = v;
+        // nobody reads C again in this launch: keep it out of the way of A and B in L2
+        __builtin_nontemporal_store(v, (i4*)(C + (size_t)(m0 + m) * p.N + n0 + c16 * 8));
       }
     }
   }

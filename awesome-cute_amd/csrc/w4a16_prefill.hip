@@ -519,7 +519,8 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     const int c16 = piece & 31;
     if (m < rows) {
       const i4 v = *(const i4*)(smem_all + m * kPitch + c16 * 16);
-      *(i4*)(C + (size_t)(m0 + m) * p.N + kPfTileN * tn + c16 * 8) = v;
+      // nobody reads C again in this launch: keep it out of the way of A and B in L2
+      __builtin_nontemporal_store(v, (i4*)(C + (size_t)(m0 + m) * p.N + kPfTileN * tn + c16 * 8));
     }
   }
   W4A16_PF_TEXIT
