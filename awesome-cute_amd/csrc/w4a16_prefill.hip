@@ -336,7 +336,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // each staging register is written to LDS (slab cs+1) and then requested
   // again (slab cs+2), so every load has a whole stage to arrive.
   auto stage_traffic = [&](int m, int ring_next, int s_next2) {
-    constexpr int kPerA = 5;  // four dword writes and the reload of one register
+    constexpr int kPerA = 3;  // two pairs of dword writes and the reload of one register
     constexpr int kBegin = 4 * RB - (HB * kPerA + 2 * 2);
     const int x = m - kBegin;
     if (x < 0) return;
@@ -348,9 +348,11 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     const int inv = sg < s_end ? 0 : kOobPf;
     if (x < HB * kPerA) {
       const int i = x / kPerA, g = x % kPerA;
-      if (g < 4)
-        *(int*)(base + a_wr + g * kPlane + i * 32 * 16) = areg[i][g];
-      else
+      if (g < 2) {
+        // two planes per slot: the pair becomes one ds_write2st64_b32
+        *(int*)(base + a_wr + (2 * g) * kPlane + i * 32 * 16) = areg[i][2 * g];
+        *(int*)(base + a_wr + (2 * g + 1) * kPlane + i * 32 * 16) = areg[i][2 * g + 1];
+      } else
         areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
     } else {
       const int y = x - HB * kPerA, i = y >> 1;
