@@ -192,6 +192,45 @@ def test_back_to_back_launches_share_scratch(env):
         assert not ws.any().item()
 
 
+def test_two_streams_run_side_by_side(env):
+    """GEMMs on two streams at the same time: each stream has its own partial-sum
+    scratch, so neither sees the other's.  Shared column tiles (streaming kernel)
+    and k slices (prefill kernel) on both; every result equals the one the same
+    call gives alone, bit for bit."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    shapes = [(4, 4096, 4096, 41), (100, 1024, 2048, 42), (16, 2048, 8192, 43), (300, 512, 4096, 44)]
+    probs = []
+    for (m, n, k, seed) in shapes:
+        A, q, s, B, sp = O.make_problem(m, n, k, 128, seed)
+        probs.append((n, torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev),
+                      torch.from_numpy(sp).to(dev)))
+
+    def run_all(stream, rounds):
+        outs = []
+        with torch.cuda.stream(stream):
+            for r in range(rounds):
+                for n, dA, dB, ds in probs:
+                    dC = torch.zeros((dA.shape[0], n), dtype=torch.half, device=dev)
+                    ws = torch.zeros(n // 128 * 16, dtype=torch.int, device=dev)
+                    marlin.mul(dA, dB, dC, ds, ws)
+                    outs.append((dC, ws))
+        return outs
+
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    alone = run_all(s1, 1)
+    torch.cuda.synchronize()
+    a = run_all(s1, 6)  # no synchronisation: the two streams' launches overlap
+    b = run_all(s2, 6)
+    torch.cuda.synchronize()
+    for outs in (a, b):
+        for i, (dC, ws) in enumerate(outs):
+            want = alone[i % len(probs)][0]
+            assert torch.equal(dC, want), (i, shapes[i % len(probs)])
+            assert not ws.any().item()
+
+
 @pytest.mark.parametrize("m", [17, 31, 32, 33, 47, 48, 49, 63, 64])
 @pytest.mark.parametrize("groupsize", [128, -1])
 def test_lds_ring_row_counts(env, m, groupsize):

@@ -138,6 +138,27 @@ def test_back_to_back_calls_share_the_scratch(env):
     close(outs[0][1].cpu().numpy(), O.dense_gemm_tn(A2, B2))
 
 
+def test_two_streams_run_side_by_side(env):
+    """Stream-K launches on two streams at once: each stream has its own partial-sum
+    buffer and tile counters; every result equals the one the same call gives alone."""
+    torch, streamk = env
+    dev = torch.device("cuda:0")
+    A1, B1 = inputs(700, 768, 1024, 3)
+    A2, B2 = inputs(256, 512, 4096, 4)
+    d = [torch.from_numpy(x).to(dev) for x in (A1, B1, A2, B2)]
+    alone = (streamk.gemm(d[0], d[1]), streamk.gemm(d[2], d[3]))
+    torch.cuda.synchronize()
+    outs = []
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for _ in range(4):
+        for st in streams:
+            with torch.cuda.stream(st):
+                outs.append((streamk.gemm(d[0], d[1]), streamk.gemm(d[2], d[3])))
+    torch.cuda.synchronize()
+    for c1, c2 in outs:
+        assert torch.equal(c1, alone[0]) and torch.equal(c2, alone[1])
+
+
 def test_degenerate_sizes_and_errors(env):
     torch, streamk = env
     dev = torch.device("cuda:0")
