@@ -231,6 +231,44 @@ def test_two_streams_run_side_by_side(env):
             assert not ws.any().item()
 
 
+def test_two_host_threads_two_streams(env):
+    """Two host threads, each with a stream of its own, call the library at the same time
+    (ctypes releases the interpreter lock during a call): the per-device state behind the
+    C ABI is locked, and both get the results a single thread gets."""
+    import threading
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    A, q, s, B, sp = O.make_problem(8, 2048, 4096, 128, 51)
+    dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+    want = torch.zeros((8, 2048), dtype=torch.half, device=dev)
+    ws0 = torch.zeros(2048 // 128 * 16, dtype=torch.int, device=dev)
+    marlin.mul(dA, dB, want, ds, ws0)
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker():
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                ws = torch.zeros(2048 // 128 * 16, dtype=torch.int, device=dev)
+                outs = [torch.zeros((8, 2048), dtype=torch.half, device=dev) for _ in range(40)]
+                for dC in outs:
+                    marlin.mul(dA, dB, dC, ds, ws)
+                st.synchronize()
+                for dC in outs:
+                    assert torch.equal(dC, want)
+                assert not ws.any().item()
+        except Exception as e:  # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker) for _ in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 @pytest.mark.parametrize("m", [17, 31, 32, 33, 47, 48, 49, 63, 64])
 @pytest.mark.parametrize("groupsize", [128, -1])
 def test_lds_ring_row_counts(env, m, groupsize):
