@@ -172,10 +172,18 @@ def cpu_baseline(O, name, budget_s=12.0):
         if dt >= budget_s or reps >= 200:
             break
     per = dt / reps
+    # the same on one core, a few repetitions
+    reps1, t1 = 0, time.perf_counter()
+    while reps1 < 3 or (time.perf_counter() - t1 < 3.0 and reps1 < 20):
+        O.gemm(A, B, sp, N, g, threads=1)
+        reps1 += 1
+    per1 = (time.perf_counter() - t1) / reps1
     return {"value": (K * N // 2) / per / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{reps} full GEMMs of {name} (M={M} N={N} K={K} group={g}), "
                       f"{per * 1e3:.1f} ms each, dequantise + fp32 GEMM, OpenMP",
-            "tflops": 2.0 * M * N * K / per / 1e12}
+            "tflops": 2.0 * M * N * K / per / 1e12,
+            "one_core": {"value": (K * N // 2) / per1 / 1e9, "unit": "GB/s", "cores": 1,
+                         "sample": f"{reps1} GEMMs, {per1 * 1e3:.1f} ms each"}}
 
 
 def main():
