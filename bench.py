@@ -48,8 +48,8 @@ SHAPES = {
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this pool); the summaries are under
 # profiles/.  None for workloads not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "decode": int((4766.7 * 2.0 + 337.5) * 1024),
-    "prefill": int((43110.1 * 2.0 + 18432.0) * 1024),
+    "decode": int((4756.5 * 2.0 + 273.0) * 1024),
+    "prefill": int((33371.5 * 2.0 + 16385.3) * 1024),
 }
 
 
