@@ -531,7 +531,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       for (int base = 0; base < n_mine; base += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) {
-          compute(d);  // a granule past the end is all zeros and adds nothing
+          // the slots past the end hold zeros: skip their arithmetic (the loads
+          // are still issued, so the load counter stays exact)
+          if (base + d < n_mine) compute(d);
           if (base + d == 0) { W4A16_STAMP(2) }
           issue(d, my_tile, ikq, base + d + DEPTH < n_mine);
           ikq += 4;
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
             clear_acc();
           }
         }
-        compute(d);  // a granule past the end is all zeros and adds nothing
+        if (i < n_mine) compute(d);  // the slots past the end hold zeros
         if (i == 0) { W4A16_STAMP(2) }
         ckq += 4;
         while (ckq >= KG) {
