@@ -388,6 +388,11 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       const int cs = s + u;
+      // an odd count of stages: nothing is left for the second copy of the last
+      // turn (the count is the same for every wave of the workgroup).  Only
+      // with 128-row tiles: with 64 the exit costs the loop more than the
+      // stage of zeros that it saves.
+      if (RB == 8 && u == 1 && cs >= stages) break;
       const int ring_next = ring == kPfRing - 1 ? 0 : ring + 1;
       const char* cur = smem + ring * kPfStageBytes;
       const char* nxt = smem + ring_next * kPfStageBytes;
