@@ -145,39 +145,20 @@ std::atomic<int> g_force_kernel{0};
 
 // Slices of the k range per prefill tile.  A slice must be at least 256 deep
 // (two 64-deep stages for each half of the workgroup) and the tile counters
-// and partial-sum slots must fit.  Measured (m = 64 ... 1024, n, k in {4096,
-// 11008, 28672 x 8192}): filling the CUs pays up to four slices; more slices
-// only add partial-sum traffic.
+// and partial-sum slots must fit.
 std::atomic<int> g_force_k_slices{0};
 // 0 = choose by cost, 64 or 128 = rows of C per prefill workgroup; set by
 // marlin_amd_force_tile_rows (tests and tools)
 std::atomic<int> g_force_tile_rows{0};
 
-int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
-  int most = k / 256;
-  if (most > 8) most = 8;
-  while (most > 1 && (size_t)tiles * most * tile_rows * 256 * 4 > kPartialBytes) --most;
-  if (most < 1 || tiles > kMaxPrefillTiles) return 1;
-  const int force = g_force_k_slices.load(std::memory_order_relaxed);
-  if (force > 0) return force < most ? force : most;
-  int s = cus / tiles;
-  if (s > 4) s = 4;
-  if (s > most) s = most;
-  return s < 1 ? 1 : s;
-}
-
-// Either kernel can do any problem whose n is a multiple of 256: the prefill
-// kernel once, or the streaming kernel once per 64 rows, reading the weights
-// again every time.  Costs in us, fitted to measurements on MI355X.
-//
-// Prefill: a full-depth tile takes 6 + 0.0130 k with 128 rows and 5 + 0.0080 k
-// with 64 (every unpacked weight then meets four row blocks instead of eight,
-// so a 64-row tile costs more than half of a 128-row one) when the launch
-// fills the CUs; k slices divide that and add their exchange, 3 + 2 s (128
-// rows: 128 KiB of partial sums per workgroup) or 3 + 1.5 s (64 rows).
-double prefill_cost_rows(int m, int n, int k, int cus, int tile_rows) {
-  const int tiles = ceil_div(m, tile_rows) * (n / 256);
-  const int s = prefill_k_slices(tiles, tile_rows, k, cus);
+// Cost in us of the prefill kernel with `tiles` tiles of tile_rows rows cut into
+// s slices, fitted to measurements on MI355X.  A full-depth tile takes
+// 6 + 0.0130 k with 128 rows and 5 + 0.0080 k with 64 (every unpacked weight
+// then meets four row blocks instead of eight, so a 64-row tile costs more than
+// half of a 128-row one) when the launch fills the CUs; k slices divide that
+// and add their exchange, 3 + 2 s (128 rows: 128 KiB of partial sums per
+// workgroup) or 3 + 1.5 s (64 rows).
+double prefill_cost_slices(int tiles, int tile_rows, int k, int cus, int s) {
   // more workgroups than CUs run in rounds, the last of which is faster the
   // emptier it is: half way between whole rounds and the plain ratio fits
   // (N = K = 4096, M = 3072: 384 tiles of 128 rows, 102.7 us, where one round
@@ -190,6 +171,40 @@ double prefill_cost_rows(int m, int n, int k, int cus, int tile_rows) {
   const double tile = (tile_rows == 64 ? 5.0 + 0.0080 * k : 6.0 + 0.0130 * k) * fill;
   const double exchange = s > 1 ? 3.0 + (tile_rows == 64 ? 1.5 : 2.0) * s : 0.0;
   return rounds * (tile / s + exchange);
+}
+
+// Slices of the k range per tile: the cheapest count among those that keep
+// the launch within one workgroup per CU, slices at least 256 deep, and the
+// partial sums and tile counters within the scratch buffer.  Up to eight; in
+// practice four, six where k is deep (N = 4096, K = 11008, M = 128: 24.8 us
+// with six against 26.9 with four).
+int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
+  int most = k / 256;
+  if (most > 8) most = 8;
+  while (most > 1 && (size_t)tiles * most * tile_rows * 256 * 4 > kPartialBytes) --most;
+  if (most < 1 || tiles > kMaxPrefillTiles) return 1;
+  const int force = g_force_k_slices.load(std::memory_order_relaxed);
+  if (force > 0) return force < most ? force : most;
+  if (most > cus / tiles) most = cus / tiles;
+  int best = 1;
+  double best_cost = prefill_cost_slices(tiles, tile_rows, k, cus, 1);
+  for (int s = 2; s <= most; s++) {
+    const double c = prefill_cost_slices(tiles, tile_rows, k, cus, s);
+    if (c < best_cost) {
+      best = s;
+      best_cost = c;
+    }
+  }
+  return best;
+}
+
+// Either kernel can do any problem whose n is a multiple of 256: the prefill
+// kernel once, or the streaming kernel once per 64 rows, reading the weights
+// again every time.
+double prefill_cost_rows(int m, int n, int k, int cus, int tile_rows) {
+  const int tiles = ceil_div(m, tile_rows) * (n / 256);
+  return prefill_cost_slices(tiles, tile_rows, k, cus,
+                             prefill_k_slices(tiles, tile_rows, k, cus));
 }
 
 // Rows of C per prefill workgroup.  64-row tiles are twice as many, so they

@@ -190,14 +190,15 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
 
 def test_kernel_choice_by_cost(marlin):
     """Few rows go through the streaming kernel, many through the prefill
-    kernel, whose k range is cut into up to four slices while tiles alone would
-    leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
+    kernel, whose k range is cut into slices (the cheapest count, at most eight)
+    while tiles alone would leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
     so do more rows while twice as many tiles save k slices.  The knobs override
     the choice."""
     for m, n, k, kernel, slices, rows in [
             (1, 4096, 4096, 1, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
             (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 2, 4, 64),
             (128, 4096, 4096, 2, 4, 64), (512, 4096, 4096, 2, 2, 64),
+            (128, 4096, 11008, 2, 6, 64), (640, 4096, 11008, 2, 3, 128),
             (512, 4096, 11008, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
             (1536, 4096, 4096, 2, 1, 128), (2048, 4096, 4096, 2, 1, 128)]:
         rc, p = marlin.plan(m, n, k, 128)
