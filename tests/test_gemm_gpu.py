@@ -379,6 +379,25 @@ def test_llama7b_shapes(env, m, k, n):
     check(env, m, n, k, -1, seed=k + n + m, thread_k=128, thread_n=128)
 
 
+@pytest.mark.parametrize("m,n,k,g", [(128, 4096, 11008, 128), (160, 4096, 11008, -1),
+                                     (96, 5120, 13568, 128), (320, 4096, 11008, 128)])
+def test_mid_rows_deep_k_planned_slices(env, m, n, k, g):
+    """Between decode and prefill over a deep k range the host cuts the tiles
+    into more than four k slices (or three, not a power of two); oracle on a
+    column slice, GPU on the whole shape, and twice the same bits."""
+    torch, marlin = env
+    rc, plan = marlin.plan(m, n, k, g)
+    assert rc == 0 and plan["kernel"] == 2 and plan["k_slices"] in (3, 5, 6), plan
+    A, q, s, B, sp = O.make_problem(m, n, k, g, seed=m + k)
+    C = gpu_gemm(env, A, B, sp, n)
+    for c0 in (0, n - 256):
+        Bs = np.ascontiguousarray(B[:, 2 * c0:2 * (c0 + 256)])
+        ss = np.ascontiguousarray(sp[:, c0:c0 + 256])
+        r = O.compare(C[:, c0:c0 + 256], O.gemm(A, Bs, ss, 256, g))
+        assert r.max_abs_err <= TOL * r.max_abs_ref, (c0, r.max_abs_err, r.max_abs_ref)
+    assert np.array_equal(gpu_gemm(env, A, B, sp, n).view(np.uint16), C.view(np.uint16))
+
+
 def test_config4_prefill_rows_sample(env):
     """M=2048, N=K=4096: the oracle checks a sample of rows (the full product
     is 69 GFLOP on the CPU); the GPU computes all of them."""
