@@ -379,6 +379,40 @@ def test_llama7b_shapes(env, m, k, n):
     check(env, m, n, k, -1, seed=k + n + m, thread_k=128, thread_n=128)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_shapes_kernels_and_knobs(env, seed):
+    """Seeded random draws over row counts around every row-block and tile
+    boundary, widths, depths, both scale modes, either kernel, both tile
+    heights and odd workgroup hints: each within tolerance of the oracle, C
+    overwritten everywhere (it starts at 9), workspace handed back zeroed."""
+    torch, marlin = env
+    rng = np.random.default_rng(seed)
+    for case in range(14):
+        g = int(rng.choice([128, -1]))
+        M = int(rng.choice([1, 2, 5, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 70, 100, 128,
+                            129, 200, 300, 513]))
+        N = (256 * int(rng.integers(1, 20)) if M > 16 or rng.random() < 0.5
+             else 128 * int(rng.integers(1, 40)))
+        K = 128 * int(rng.integers(1, 40))
+        if K == 128 and g == 128:
+            K = 256
+        forced = int(rng.choice([0, 0, 1, 2])) if N % 256 == 0 else 0
+        rows = int(rng.choice([0, 64, 128]))
+        sms = int(rng.choice([-1, -1, -1, 7, 64, 100, 256, 300, 1000]))
+        assert marlin.check(M, N, K, g) == 0
+        print(f"  case {seed}/{case}: forced kernel {forced}, tile rows {rows}", flush=True)
+        marlin.force_kernel(forced)
+        marlin.force_tile_rows(rows)
+        try:
+            A, q, s, B, sp = O.make_problem(M, N, K, g, 1000 * seed + case)
+            C = gpu_gemm(env, A, B, sp, N, sms=sms, C_fill=9.0)
+        finally:
+            marlin.force_kernel(0)
+            marlin.force_tile_rows(0)
+        r = O.compare(C, O.gemm(A, B, sp, N, g))
+        assert r.max_abs_err <= TOL * r.max_abs_ref, (M, N, K, g, forced, rows, sms, r.max_abs_err)
+
+
 @pytest.mark.parametrize("m,n,k,g", [(128, 4096, 11008, 128), (160, 4096, 11008, -1),
                                      (96, 5120, 13568, 128), (320, 4096, 11008, 128)])
 def test_mid_rows_deep_k_planned_slices(env, m, n, k, g):
