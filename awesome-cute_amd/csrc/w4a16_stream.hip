@@ -212,13 +212,9 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
                       : smem + wave * (MB * 2048);
   const int a_wr = ((lane >> 2) * 4 + ax) * 4;
   const int a_rd = kDmaA ? 16 * nu + 4 * kg : (kg * 16 + nu) * 16;
-  if constexpr (kDmaA) {
-    // A granule that does not exist multiplies zero weights with whatever its
-    // ring slot holds, so the ring must never hold NaN or Inf bit patterns.
-    for (int o = lane * 16; o < Lds::kRingBytesPerWave; o += 1024)
-      *(i4*)(lds_a + o) = (i4){0, 0, 0, 0};
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): zeros are in before the first ring load
-  }
+  // (The ring starts with whatever LDS held: a slot is only ever read after a
+  // granule that exists was loaded into it -- the arithmetic on slots past the
+  // end of the run is skipped below.)
 
   const DequantConsts dc;
 
