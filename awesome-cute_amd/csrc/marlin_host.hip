@@ -222,23 +222,76 @@ double prefill_cost(int m, int n, int k, int cus) {
   return prefill_cost_rows(m, n, k, cus, prefill_tile_rows(m, n, k, cus));
 }
 
-double stream_cost(int m, int n, int k) {
-  const double mb = 0.5e-6 * n * k;  // MB of packed weights, read once per pass
-  // a pass over 49-64 rows (4 row blocks); the slope flattens for big problems
-  const double full = mb <= 22.5 ? 9.8 + 0.60 * mb : 23.3 + 0.25 * (mb - 22.5);
+// The streaming kernel's split of the granule sequence over the compute units
+// for `mb` row blocks.  Measured on MI355X: a split that keeps every workgroup
+// inside one column tile (or gives it whole tiles) costs about 0.1 us x row
+// blocks per granule of the longest workgroup; a split that leaves workgroups
+// straddling tile boundaries is several us slower (a second exchange per
+// workgroup, and workgroups that read different weight rows at the same
+// time), about 1 + 2.5 x row blocks us.  Candidates: every tile cut into c
+// nearly equal runs (c tiles' worth of workgroups <= CUs), whole tiles per
+// workgroup, and the evenly balanced uniform split.
+struct StreamSplit {
+  int gpb;        // granules of the longest workgroup
+  int wpt;        // workgroups per column tile, or 0 for the uniform form
+  bool straddle;  // workgroups cross tile boundaries
+};
+StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
+  const int NT = n / kTileN;
+  const int KG = k / kGranuleK;
+  const int total = NT * KG;
+  const double per_granule = 0.1 * mb, straddle = 1.0 + 2.5 * mb;
+  StreamSplit sp;
+  sp.gpb = ceil_div(total, cus);
+  sp.wpt = 0;
+  sp.straddle = !(sp.gpb % KG == 0 || KG % sp.gpb == 0);
+  double best_cost = per_granule * sp.gpb + (sp.straddle ? straddle : 0.0);
+  for (int c = 1; c <= KG && NT * c <= cus; c++) {
+    const int g = ceil_div(KG, c);
+    const double cost = per_granule * g;
+    if (cost < best_cost + 1e-9) {  // on a tie the one-tile form: its kernel is leaner
+      sp.gpb = g;
+      sp.wpt = c;
+      sp.straddle = false;
+      best_cost = cost;
+    }
+  }
+  for (int mult = 2; mult * KG <= total; mult++) {
+    const int g = mult * KG;
+    if (ceil_div(total, g) > cus) continue;  // more workgroups than CUs never paid off
+    const double cost = per_granule * g;
+    if (cost < best_cost - 1e-9) {
+      sp.gpb = g;
+      sp.wpt = 0;
+      sp.straddle = false;
+      best_cost = cost;
+    }
+  }
+  return sp;
+}
+
+// Fitted time (us) of the streaming kernel: a pass over 49-64 rows takes
+// 12.1 + 0.285 per granule of the longest workgroup (N=K=4096: 8 granules,
+// 13.9; N=11008, K=4096 or 8192^2: 32, 20.3-21.2; N=28672, K=8192: 128, 48),
+// fewer rows a share of that, up to 16 rows 5.1 + 0.16 per granule.
+double stream_cost(int m, int n, int k, int cus) {
+  const StreamSplit s4 = choose_stream_split(4, n, k, cus);
+  const double full = 12.1 + 0.285 * s4.gpb + (s4.straddle ? 11.0 : 0.0);
   const int tail = m % kStreamMaxRows;
   double t = (m / kStreamMaxRows) * full;
-  if (tail > 16)
+  if (tail > 16) {
     t += full * (tail > 48 ? 1.0 : tail > 32 ? 0.9 : 0.65);
-  else if (tail > 0)
-    t += 5.0 + 0.25 * mb;
+  } else if (tail > 0) {
+    const StreamSplit s1 = choose_stream_split(1, n, k, cus);
+    t += 5.1 + 0.16 * s1.gpb + (s1.straddle ? 3.5 : 0.0);
+  }
   return t;
 }
 
 bool prefer_prefill(int m, int n, int k, int cus) {
   // no measurement favours 64-row prefill tiles below four row blocks
   if (m <= 48) return false;
-  return prefill_cost(m, n, k, cus) <= stream_cost(m, n, k);
+  return prefill_cost(m, n, k, cus) <= stream_cost(m, n, k, cus);
 }
 
 Plan make_plan(int m, int n, int k, int sms, int cus) {
@@ -265,45 +318,13 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   if (sms > 0) {
     pl.sp = make_stream_plan(n, k, sms > kMaxStreamGrid ? kMaxStreamGrid : sms);
   } else {
-    // Measured on MI355X: a split that keeps every workgroup inside one
-    // column tile (or gives it whole tiles) costs about 0.1 us x row blocks
-    // per granule of the longest workgroup; a split that leaves workgroups
-    // straddling tile boundaries is several us slower (a second exchange per
-    // workgroup, and workgroups that read different weight rows at the same
-    // time), about 1 + 2.5 x row blocks us.  Candidates: every tile cut into
-    // c nearly equal runs (c tiles' worth of workgroups <= CUs), whole tiles
-    // per workgroup, and the evenly balanced uniform split.
     const int mb = ceil_div(m < kStreamMaxRows ? m : kStreamMaxRows, 16);
-    const int NT = n / kTileN;
-    const int KG = k / kGranuleK;
-    const int total = NT * KG;
-    const double per_granule = 0.1 * mb, straddle = 1.0 + 2.5 * mb;
-    int best = ceil_div(total, cus), best_wpt = 0;
-    double best_cost = per_granule * best + ((best % KG == 0 || KG % best == 0) ? 0.0 : straddle);
-    for (int c = 1; c <= KG && NT * c <= cus; c++) {
-      const int g = ceil_div(KG, c);
-      const double cost = per_granule * g;
-      if (cost < best_cost + 1e-9) {  // on a tie the one-tile form: its kernel is leaner
-        best = g;
-        best_wpt = c;
-        best_cost = cost;
-      }
-    }
-    for (int mult = 2; mult * KG <= total; mult++) {
-      const int g = mult * KG;
-      if (ceil_div(total, g) > cus) continue;  // more workgroups than CUs never paid off
-      const double cost = per_granule * g;
-      if (cost < best_cost - 1e-9) {
-        best = g;
-        best_wpt = 0;
-        best_cost = cost;
-      }
-    }
-    pl.sp.NT = NT;
-    pl.sp.KG = KG;
-    pl.sp.gpb = best;
-    pl.sp.wpt = best_wpt;
-    pl.sp.grid = best_wpt > 0 ? NT * best_wpt : ceil_div(total, best);
+    const StreamSplit split = choose_stream_split(mb, n, k, cus);
+    pl.sp.NT = n / kTileN;
+    pl.sp.KG = k / kGranuleK;
+    pl.sp.gpb = split.gpb;
+    pl.sp.wpt = split.wpt;
+    pl.sp.grid = split.wpt > 0 ? pl.sp.NT * split.wpt : ceil_div(pl.sp.NT * pl.sp.KG, split.gpb);
   }
   pl.grid = pl.sp.grid;
   pl.launches = ceil_div(m, kStreamMaxRows);
