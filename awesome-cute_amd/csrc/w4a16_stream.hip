@@ -597,12 +597,13 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   W4A16_STAMP(8)
 }
 
-// ring depth of the deep variant: a workgroup inside one tile can afford four
-// slots for any row-block count (see StreamLds), the other form three from
-// three row blocks on
+// Ring depth of the deep variant.  Three granules in flight per wave measured
+// faster than four for every row-block count (M=16: N=11008 10.3 -> 9.9 us,
+// K=11008 10.4 -> 9.6; 64 rows at K=11008 21.2 -> 18.4), and eight slower
+// still: the more requests a CU has in flight, the slower the stream.
 template <int MB, bool ONE_TILE>
 constexpr int deep_ring() {
-  return (ONE_TILE || MB <= 2) ? 4 : 3;
+  return 3;
 }
 
 template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
