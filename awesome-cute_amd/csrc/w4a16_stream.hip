@@ -600,10 +600,12 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 // Ring depth of the deep variant.  Three granules in flight per wave measured
 // faster than four for every row-block count (M=16: N=11008 10.3 -> 9.9 us,
 // K=11008 10.4 -> 9.6; 64 rows at K=11008 21.2 -> 18.4), and eight slower
-// still: the more requests a CU has in flight, the slower the stream.
+// still: the more requests a CU has in flight, the slower the stream.  With
+// two row blocks two are better again (M=32, N=11008: 12.7 -> 12.4 us), with
+// three and four they are 2-5 % worse.
 template <int MB, bool ONE_TILE>
 constexpr int deep_ring() {
-  return 3;
+  return MB == 2 ? 2 : 3;
 }
 
 template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
