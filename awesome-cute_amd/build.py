@@ -10,7 +10,9 @@ LIB = os.path.join(HERE, "libmarlin_amd.so")
 # default register split produces around every MFMA.
 SOURCES = {
     "marlin_host.hip": [],
+    "scratch_pool.hip": [],
     "w4a16_stream.hip": [],
+    "w4a16_probe.hip": [],
     "w4a16_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "f16_streamk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }

@@ -37,6 +37,7 @@
 #include <vector>
 
 #include "../../include/streamk_amd.h"
+#include "scratch_pool.hpp"
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
@@ -47,7 +48,6 @@ constexpr int kDnTile = 256;     // columns of a tile of C, and rows of the larg
 constexpr int kDnStageK = 64;    // k depth of a stage (two MFMA k steps)
 constexpr int kDnRing = 2;       // slabs in LDS
 constexpr int kDnOob = (int)0x80000000;
-constexpr int kDnPartBytes = kDnTile * kDnTile * 4;  // fp32 partial sums of one slice (large tile)
 
 // LDS geometry for tiles of TM rows (256, or 128 when the large tiles are too
 // few for the compute units): a slab is TM rows of A and 256 rows of B
@@ -418,8 +418,6 @@ namespace {
 using namespace w4a16;
 
 constexpr int kDnMaxDevices = 16;
-constexpr size_t kDnPartialBytes = (size_t)kDnMaxSlots * kDnPartBytes;
-constexpr size_t kDnScratchBytes = kDnPartialBytes + (size_t)kDnMaxSlots * sizeof(int);
 
 thread_local char g_dn_error[256] = "";
 
@@ -427,16 +425,12 @@ void dn_set_error(hipError_t e, const char* what) {
   snprintf(g_dn_error, sizeof(g_dn_error), "%s: %s", what, hipGetErrorString(e));
 }
 
-// one buffer of partial sums and tile counters per (device, stream), kept
-// until the process ends; the counters are zero whenever no launch is in flight
-struct DnScratch {
-  hipStream_t stream;
-  float* ptr;
-};
+// Partial sums and tile counters of the stream-K tiles come from the scratch
+// pool that the W4A16 path uses too: one buffer per (device, stream), sized by
+// the launches that need it.
 struct DnDevice {
   int cus = 0;
   bool configured = false;
-  std::vector<DnScratch> scratch;
 };
 std::mutex g_dn_mu;
 DnDevice g_dn[kDnMaxDevices];
@@ -520,7 +514,6 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
   }
   rc = STREAMK_ERR_RUNTIME;
   do {
-    float* scratch = nullptr;
     int cus = 0;
     {
       std::lock_guard<std::mutex> lk(g_dn_mu);
@@ -546,24 +539,16 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
         }
         d.configured = true;
       }
-      for (const DnScratch& s : d.scratch)
-        if (s.stream == stream) scratch = s.ptr;
-      if (!scratch) {
-        e = hipMalloc((void**)&scratch, kDnScratchBytes);
-        if (e != hipSuccess) {
-          dn_set_error(e, "hipMalloc(scratch)");
-          break;
-        }
-        e = hipMemset((char*)scratch + kDnPartialBytes, 0, kDnScratchBytes - kDnPartialBytes);
-        if (e != hipSuccess) {
-          dn_set_error(e, "hipMemset(scratch)");
-          (void)hipFree(scratch);
-          break;
-        }
-        d.scratch.push_back({stream, scratch});
-      }
     }
     const DnPlan pl = dn_plan(m, n, k, cus);
+    // only a launch with stream-K tiles exchanges anything
+    ScratchView view = {nullptr, nullptr};
+    if (pl.sk_tiles > 0 &&
+        !scratch_acquire(dev, stream,
+                         (size_t)pl.sk_tiles * pl.ksplit * pl.tile_rows * kDnTile * 4, &view,
+                         g_dn_error, sizeof(g_dn_error)))
+      break;
+    (void)hipGetLastError();  // an earlier call's error is not this launch's
     DenseArgs a;
     a.A = A;
     a.B = B;
@@ -577,8 +562,8 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.dp_tiles = pl.dp_tiles;
     a.sk_tiles = pl.sk_tiles;
     a.ksplit = pl.ksplit;
-    a.locks = (int*)((char*)scratch + kDnPartialBytes);
-    a.scratch = scratch;
+    a.locks = view.counters;
+    a.scratch = view.partials;
     if (pl.tile_rows == 128)
       hipLaunchKernelGGL(dense_kernel<128>, dim3(pl.grid), dim3(512), DnShape<128>::kLds, stream, a);
     else
@@ -613,6 +598,8 @@ int streamk_amd_plan(int m, int n, int k, int cus, int* out) {
 void streamk_amd_tile_coord(int tile, int tiles_m, int tiles_n, int* out) {
   dn_tile_coord(tile, tiles_m, tiles_n, &out[0], &out[1]);
 }
+
+long long streamk_amd_release(int dev) { return (long long)scratch_release(dev); }
 
 const char* streamk_amd_last_error(void) { return g_dn_error; }
 

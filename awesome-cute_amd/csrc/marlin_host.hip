@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "../../include/marlin_amd.h"
+#include "scratch_pool.hpp"
 #include "w4a16_common.hpp"
 
 namespace {
@@ -29,27 +30,16 @@ void set_error(hipError_t e, const char* what) {
   snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
 }
 
-// Partial-sum scratch of the streaming kernel: one buffer per (device, stream)
-// so that GEMMs on different streams never share partial sums.  Buffers live
-// until the process ends.
-struct Scratch {
-  hipStream_t stream;
-  float* ptr;
-};
 struct DeviceState {
   int cus = 0;
-  bool configured = false;  // kernels' LDS limits raised on this device
-  std::vector<Scratch> scratch;
+  bool configured = false;          // kernels' LDS limits raised on this device
 };
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 
-constexpr size_t kPartialBytes = (size_t)2 * kMaxStreamGrid * stream_slot_bytes(4);
-// behind the partial sums: the tile counters of the prefill kernel's k slices
-// (the caller's workspace has one counter per 128 columns, too few for tiles
-// of many rows), zero whenever no launch is in flight
-constexpr int kMaxPrefillTiles = 16384;
-constexpr size_t kScratchBytes = kPartialBytes + (size_t)kMaxPrefillTiles * sizeof(int);
+// What the planner may assume about the partial-sum buffer: the pool grows up
+// to this much for one call.
+constexpr size_t kPoolPartialLimit = (size_t)64 << 20;
 
 // With `dev` current: raise the dynamic-LDS limit of the kernels that need it.
 bool configure_device(int dev) {
@@ -75,26 +65,6 @@ int device_cus(int dev) {
     g_dev[dev].cus = cus;
   }
   return g_dev[dev].cus;
-}
-
-float* scratch_for(int dev, hipStream_t stream) {
-  std::lock_guard<std::mutex> lk(g_mu);
-  for (const Scratch& s : g_dev[dev].scratch)
-    if (s.stream == stream) return s.ptr;
-  float* p = nullptr;
-  hipError_t e = hipMalloc((void**)&p, kScratchBytes);
-  if (e != hipSuccess) {
-    set_error(e, "hipMalloc(scratch)");
-    return nullptr;
-  }
-  e = hipMemset((char*)p + kPartialBytes, 0, kScratchBytes - kPartialBytes);
-  if (e != hipSuccess) {
-    set_error(e, "hipMemset(scratch)");
-    (void)hipFree(p);
-    return nullptr;
-  }
-  g_dev[dev].scratch.push_back({stream, p});
-  return p;
 }
 
 // Shape checks in the order the reference performs them
@@ -133,23 +103,29 @@ struct Plan {
   int grid;
   StreamPlan sp;
   int launches;
-  int ksplit;     // prefill: slices of the k range per tile
-  int tile_rows;  // prefill: rows of C per workgroup
+  int ksplit;            // prefill: slices of the k range per tile
+  int tile_rows;         // prefill: rows of C per workgroup
+  size_t partial_bytes;  // fp32 partial sums the launch exchanges through scratch (0: none)
 };
 
 constexpr int kStreamMaxRows = 64;
 
-// 0 = choose by cost, 1 = streaming kernel (in chunks of 64 rows), 2 = prefill
-// kernel; set by marlin_amd_force_kernel (tests and tools)
-std::atomic<int> g_force_kernel{0};
+// Overrides of the planner for the calling thread (tests and tools; see
+// marlin_amd_force_*): which kernel (0 = by cost, 1 = streaming in chunks of
+// 64 rows, 2 = prefill), slices of the k range per prefill tile (0 = by cost),
+// rows of C per prefill workgroup (0 = by cost, 64 or 128).
+struct Force {
+  int kernel = 0, k_slices = 0, tile_rows = 0;
+};
+thread_local Force t_force;
 
-// Slices of the k range per prefill tile.  A slice must be at least 256 deep
-// (two 64-deep stages for each half of the workgroup) and the tile counters
-// and partial-sum slots must fit.
-std::atomic<int> g_force_k_slices{0};
-// 0 = choose by cost, 64 or 128 = rows of C per prefill workgroup; set by
-// marlin_amd_force_tile_rows (tests and tools)
-std::atomic<int> g_force_tile_rows{0};
+// What a plan is made for: the device's compute units, the room for partial
+// sums, and the thread's overrides.
+struct PlanCtx {
+  int cus;
+  size_t partial_limit;
+  Force force;
+};
 
 // Cost in us of the prefill kernel with `tiles` tiles of tile_rows rows cut into
 // s slices, fitted to measurements on MI355X.  A full-depth tile takes
@@ -174,22 +150,22 @@ double prefill_cost_slices(int tiles, int tile_rows, int k, int cus, int s) {
 }
 
 // Slices of the k range per tile: the cheapest count among those that keep
-// the launch within one workgroup per CU, slices at least 256 deep, and the
-// partial sums and tile counters within the scratch buffer.  Up to eight; in
-// practice four, six where k is deep (N = 4096, K = 11008, M = 128: 24.8 us
-// with six against 26.9 with four).
-int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
+// the launch within one workgroup per CU, slices at least 256 deep (two
+// 64-deep stages for each half of the workgroup), and the partial sums and
+// tile counters within the scratch.  Up to eight; in practice four, six where
+// k is deep (N = 4096, K = 11008, M = 128: 24.8 us with six against 26.9 with
+// four).
+int prefill_k_slices(int tiles, int tile_rows, int k, const PlanCtx& cx) {
   int most = k / 256;
   if (most > 8) most = 8;
-  while (most > 1 && (size_t)tiles * most * tile_rows * 256 * 4 > kPartialBytes) --most;
-  if (most < 1 || tiles > kMaxPrefillTiles) return 1;
-  const int force = g_force_k_slices.load(std::memory_order_relaxed);
-  if (force > 0) return force < most ? force : most;
-  if (most > cus / tiles) most = cus / tiles;
+  while (most > 1 && (size_t)tiles * most * tile_rows * 256 * 4 > cx.partial_limit) --most;
+  if (most < 1 || tiles > kMaxCounters) return 1;
+  if (cx.force.k_slices > 0) return cx.force.k_slices < most ? cx.force.k_slices : most;
+  if (most > cx.cus / tiles) most = cx.cus / tiles;
   int best = 1;
-  double best_cost = prefill_cost_slices(tiles, tile_rows, k, cus, 1);
+  double best_cost = prefill_cost_slices(tiles, tile_rows, k, cx.cus, 1);
   for (int s = 2; s <= most; s++) {
-    const double c = prefill_cost_slices(tiles, tile_rows, k, cus, s);
+    const double c = prefill_cost_slices(tiles, tile_rows, k, cx.cus, s);
     if (c < best_cost) {
       best = s;
       best_cost = c;
@@ -201,25 +177,24 @@ int prefill_k_slices(int tiles, int tile_rows, int k, int cus) {
 // Either kernel can do any problem whose n is a multiple of 256: the prefill
 // kernel once, or the streaming kernel once per 64 rows, reading the weights
 // again every time.
-double prefill_cost_rows(int m, int n, int k, int cus, int tile_rows) {
+double prefill_cost_rows(int m, int n, int k, const PlanCtx& cx, int tile_rows) {
   const int tiles = ceil_div(m, tile_rows) * (n / 256);
-  return prefill_cost_slices(tiles, tile_rows, k, cus,
-                             prefill_k_slices(tiles, tile_rows, k, cus));
+  return prefill_cost_slices(tiles, tile_rows, k, cx.cus,
+                             prefill_k_slices(tiles, tile_rows, k, cx));
 }
 
 // Rows of C per prefill workgroup.  64-row tiles are twice as many, so they
 // need fewer k slices to fill the CUs (or none), which wins while the problem
 // is small: at N = K = 4096 up to about 512 rows (M = 128: 16.0 against
 // 21.9 us), at N = 4096, K = 11008 up to 256 (27.5 against 38.9 us at M = 128).
-int prefill_tile_rows(int m, int n, int k, int cus) {
-  const int force = g_force_tile_rows.load(std::memory_order_relaxed);
-  if (force == 64 || force == 128) return force;
+int prefill_tile_rows(int m, int n, int k, const PlanCtx& cx) {
+  if (cx.force.tile_rows == 64 || cx.force.tile_rows == 128) return cx.force.tile_rows;
   if (m <= 64) return 64;
-  return prefill_cost_rows(m, n, k, cus, 64) < prefill_cost_rows(m, n, k, cus, 128) ? 64 : 128;
+  return prefill_cost_rows(m, n, k, cx, 64) < prefill_cost_rows(m, n, k, cx, 128) ? 64 : 128;
 }
 
-double prefill_cost(int m, int n, int k, int cus) {
-  return prefill_cost_rows(m, n, k, cus, prefill_tile_rows(m, n, k, cus));
+double prefill_cost(int m, int n, int k, const PlanCtx& cx) {
+  return prefill_cost_rows(m, n, k, cx, prefill_tile_rows(m, n, k, cx));
 }
 
 // The streaming kernel's split of the granule sequence over the compute units
@@ -240,6 +215,7 @@ StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
   const int NT = n / kTileN;
   const int KG = k / kGranuleK;
   const int total = NT * KG;
+  if (cus > kMaxStreamGrid) cus = kMaxStreamGrid;  // the grid the kernel's slots allow
   const double per_granule = 0.1 * mb, straddle = 1.0 + 2.5 * mb;
   StreamSplit sp;
   sp.gpb = ceil_div(total, cus);
@@ -288,38 +264,41 @@ double stream_cost(int m, int n, int k, int cus) {
   return t;
 }
 
-bool prefer_prefill(int m, int n, int k, int cus) {
+bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   // no measurement favours 64-row prefill tiles below four row blocks
   if (m <= 48) return false;
-  return prefill_cost(m, n, k, cus) <= stream_cost(m, n, k, cus);
+  return prefill_cost(m, n, k, cx) <= stream_cost(m, n, k, cx.cus);
 }
 
-Plan make_plan(int m, int n, int k, int sms, int cus) {
+Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   Plan pl;
-  const int force = g_force_kernel.load(std::memory_order_relaxed);
+  const int force = cx.force.kernel;
   // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
   // whenever m > 16, by the shape contract)
   const bool prefill =
-      n % 256 == 0 && (force == 2 || (force == 0 && prefer_prefill(m, n, k, cus)));
+      n % 256 == 0 && (force == 2 || (force == 0 && prefer_prefill(m, n, k, cx)));
   pl.ksplit = 1;
   pl.tile_rows = 0;
+  pl.partial_bytes = 0;
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
-    pl.tile_rows = prefill_tile_rows(m, n, k, cus);
+    pl.tile_rows = prefill_tile_rows(m, n, k, cx);
     const int tiles = ceil_div(m, pl.tile_rows) * (n / 256);
-    pl.ksplit = prefill_k_slices(tiles, pl.tile_rows, k, cus);
+    pl.ksplit = prefill_k_slices(tiles, pl.tile_rows, k, cx);
     pl.grid = tiles * pl.ksplit;
     pl.sp = make_stream_plan(n, k, 1);
     pl.launches = 1;
+    if (pl.ksplit > 1) pl.partial_bytes = (size_t)pl.grid * pl.tile_rows * 256 * 4;
     return pl;
   }
   pl.kernel = 1;
+  const int rows = m < kStreamMaxRows ? m : kStreamMaxRows;
+  const int mb = ceil_div(rows, 16);
   if (sms > 0) {
     pl.sp = make_stream_plan(n, k, sms > kMaxStreamGrid ? kMaxStreamGrid : sms);
   } else {
-    const int mb = ceil_div(m < kStreamMaxRows ? m : kStreamMaxRows, 16);
-    const StreamSplit split = choose_stream_split(mb, n, k, cus);
+    const StreamSplit split = choose_stream_split(mb, n, k, cx.cus);
     pl.sp.NT = n / kTileN;
     pl.sp.KG = k / kGranuleK;
     pl.sp.gpb = split.gpb;
@@ -328,19 +307,73 @@ Plan make_plan(int m, int n, int k, int sms, int cus) {
   }
   pl.grid = pl.sp.grid;
   pl.launches = ceil_div(m, kStreamMaxRows);
+  // column tiles that several workgroups share are finished through one
+  // partial-sum slot per workgroup (cut tiles) or two (runs that may start and
+  // end inside a tile)
+  const bool shared = pl.sp.wpt > 0 ? pl.sp.wpt > 1 : pl.sp.gpb % pl.sp.KG != 0;
+  if (shared) pl.partial_bytes = (size_t)stream_slots(pl.sp) * stream_slot_bytes(mb);
   return pl;
+}
+
+// Enqueue the launches of plan pl with the scratch of `view` (null pointers
+// when the plan exchanges nothing through scratch).
+int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* B, void* C,
+            const void* s, int m, int n, int k, void* workspace, int groupsize, int max_par,
+            hipStream_t stream) {
+  // the caller's workspace holds at least n/128 * max_par zero ints
+  // (reference marlin_gemm.cpp:29-31, marlin_cute_kernel.cu:68); one counter
+  // per column tile is used, and the counters are spread max_par ints apart
+  // (64 bytes at the launcher's default of 16)
+  const int lock_stride = max_par > 16 ? 16 : max_par;
+  (void)hipGetLastError();  // an earlier call's error is not this launch's
+  int rc = MARLIN_OK;
+  if (pl.kernel == 2) {
+    GemmArgs a;
+    a.A = A;
+    a.B = B;
+    a.C = C;
+    a.S = s;
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.locks = view.counters;
+    a.lock_stride = 1;
+    a.scratch = view.partials;
+    a.gpb = 0;
+    a.wpt = 0;
+    rc = launch_prefill(a, groupsize != -1, pl.ksplit, pl.tile_rows, stream);
+  } else {
+    for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
+      GemmArgs a;
+      a.A = (const char*)A + (size_t)m0 * k * 2;
+      a.B = B;
+      a.C = (char*)C + (size_t)m0 * n * 2;
+      a.S = s;
+      a.M = m - m0 < kStreamMaxRows ? m - m0 : kStreamMaxRows;
+      a.N = n;
+      a.K = k;
+      a.locks = (int*)workspace;
+      a.lock_stride = lock_stride;
+      a.scratch = view.partials;
+      a.gpb = pl.sp.gpb;
+      a.wpt = pl.sp.wpt;
+      rc = launch_stream(a, groupsize != -1, pl.grid, stream);
+    }
+  }
+  if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
+  return rc;
 }
 
 int run(const void* A, const void* B, void* C, const void* s, int m, int n, int k,
         void* workspace, int groupsize, int dev, hipStream_t stream, int thread_k, int thread_n,
         int sms, int max_par) {
-  // the caller's workspace holds at least n/128 * max_par zero ints
-  // (reference marlin_gemm.cpp:29-31, marlin_cute_kernel.cu:68); one counter
-  // per column tile is used, and the counters are spread max_par ints apart
-  // (64 bytes at the launcher's default of 16)
-  const int lock_stride = max_par < 1 ? 1 : (max_par > 16 ? 16 : max_par);
   int rc = check_shape(m, n, k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || m == 0 || n == 0 || k == 0) return rc;
+  if (max_par < 1) {
+    // the tile counters live in the caller's workspace, max_par ints apart
+    snprintf(g_last_error, sizeof(g_last_error), "max_par = %d: must be at least 1", max_par);
+    return MARLIN_ERR_WORKSPACE;
+  }
   // the kernels address A, B and C with 32-bit byte offsets
   const long long lim = 0x7fffffffLL;
   if ((long long)k * n / 2 > lim || (long long)m * k * 2 > lim || (long long)m * n * 2 > lim) {
@@ -362,48 +395,19 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
     set_error(e, "hipSetDevice");
     return MARLIN_ERR_RUNTIME;
   }
-  int cus = device_cus(dev);
+  const int cus = device_cus(dev);
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0 && configure_device(dev)) {
-    Plan pl = make_plan(m, n, k, sms, cus);
-    float* scratch =
-        pl.kernel == 1 || pl.ksplit > 1 ? scratch_for(dev, stream) : nullptr;
-    if (pl.kernel == 2 && (pl.ksplit == 1 || scratch)) {
-      GemmArgs a;
-      a.A = A;
-      a.B = B;
-      a.C = C;
-      a.S = s;
-      a.M = m;
-      a.N = n;
-      a.K = k;
-      a.locks = scratch ? (int*)((char*)scratch + kPartialBytes) : nullptr;
-      a.lock_stride = 1;
-      a.scratch = scratch;
-      a.gpb = 0;
-      a.wpt = 0;
-      rc = launch_prefill(a, groupsize != -1, pl.ksplit, pl.tile_rows, stream);
-      if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
-    } else if (pl.kernel == 1 && scratch) {
-      rc = MARLIN_OK;
-      for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
-        GemmArgs a;
-        a.A = (const char*)A + (size_t)m0 * k * 2;
-        a.B = B;
-        a.C = (char*)C + (size_t)m0 * n * 2;
-        a.S = s;
-        a.M = m - m0 < kStreamMaxRows ? m - m0 : kStreamMaxRows;
-        a.N = n;
-        a.K = k;
-        a.locks = (int*)workspace;
-        a.lock_stride = lock_stride;
-        a.scratch = scratch;
-        a.gpb = pl.sp.gpb;
-        a.wpt = pl.sp.wpt;
-        rc = launch_stream(a, groupsize != -1, pl.grid, stream);
-      }
-      if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
+    const PlanCtx cx = {cus, kPoolPartialLimit, t_force};
+    const Plan pl = make_plan(m, n, k, sms, cx);
+    ScratchView view = {nullptr, nullptr};
+    bool ok = true;
+    if (pl.partial_bytes > 0) {
+      ok = scratch_acquire(dev, stream, pl.partial_bytes, &view, g_last_error,
+                           sizeof(g_last_error));
     }
+    if (ok)
+      rc = enqueue(pl, view, A, B, C, s, m, n, k, workspace, groupsize, max_par, stream);
   }
   if (prev != dev) (void)hipSetDevice(prev);
   return rc;
@@ -448,11 +452,14 @@ int marlin_mul(const void* A, const void* B, void* C, const void* s, int prob_m,
   int groupsize = s_rows == 1 ? -1 : prob_k / s_rows;
   if (groupsize != -1 && groupsize * s_rows != prob_k)
     return fail(MARLIN_ERR_GROUPS, "k=%d not compatible with %d groups.", prob_k, s_rows);
-  if (workspace_numel < (long long)(prob_n / 128) * max_par)
+  // (the reference's comparison, marlin_gemm.cpp:29-31, lets any workspace pass
+  // when max_par < 1; the tile counters need at least one int per tile)
+  const int par = max_par < 1 ? 1 : max_par;
+  if (workspace_numel < (long long)(prob_n / 128) * par)
     return fail(MARLIN_ERR_WORKSPACE, "workspace must be of size at least %d.",
-                prob_n / 128 * max_par);
+                prob_n / 128 * par);
   int rc = marlin_gemm(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream,
-                       thread_k, thread_n, sms, max_par);
+                       thread_k, thread_n, sms, par);
   if (rc == MARLIN_ERR_PROB_SHAPE)
     return fail(rc, "Problem (m=%d, n=%d, k=%d) not compatible with thread_k=%d, thread_n=%d.",
                 prob_m, prob_n, prob_k, thread_k, thread_n);
@@ -460,6 +467,7 @@ int marlin_mul(const void* A, const void* B, void* C, const void* s, int prob_m,
     return fail(rc, "No kernel implementation for thread_k=%d, thread_n=%d, groupsize=%d.",
                 thread_k, thread_n, groupsize);
   if (rc == MARLIN_ERR_RUNTIME) return fail(rc, "HIP runtime error: %s", g_last_error);
+  if (rc != MARLIN_OK) return fail(rc, "%s", g_last_error);
   return rc;
 }
 
@@ -470,10 +478,11 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int* out) {
-  for (int i = 0; i < 9; i++) out[i] = 0;
+  for (int i = 0; i < 10; i++) out[i] = 0;
   int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
-  Plan pl = make_plan(prob_m, prob_n, prob_k, sms, cus);
+  const PlanCtx cx = {cus, kPoolPartialLimit, t_force};
+  Plan pl = make_plan(prob_m, prob_n, prob_k, sms, cx);
   out[0] = pl.kernel;
   out[1] = pl.grid;
   out[2] = pl.sp.gpb;
@@ -483,27 +492,71 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[6] = pl.ksplit;
   out[7] = pl.tile_rows;
   out[8] = pl.kernel == 1 ? pl.sp.wpt : 0;
+  out[9] = (int)(pl.partial_bytes >> 10);
   return rc;
 }
 
-void marlin_amd_force_kernel(int which) {
-  g_force_kernel.store(which == 1 || which == 2 ? which : 0, std::memory_order_relaxed);
-}
+void marlin_amd_force_kernel(int which) { t_force.kernel = which == 1 || which == 2 ? which : 0; }
 
-void marlin_amd_force_k_slices(int slices) {
-  g_force_k_slices.store(slices > 0 ? slices : 0, std::memory_order_relaxed);
-}
+void marlin_amd_force_k_slices(int slices) { t_force.k_slices = slices > 0 ? slices : 0; }
 
-void marlin_amd_force_tile_rows(int rows) {
-  g_force_tile_rows.store(rows == 64 || rows == 128 ? rows : 0, std::memory_order_relaxed);
-}
+void marlin_amd_force_tile_rows(int rows) { t_force.tile_rows = rows == 64 || rows == 128 ? rows : 0; }
 
 void marlin_amd_work_order(int grid, int* out) {
   for (int b = 0; b < grid; b++) out[b] = xcd_work_index(b, grid);
 }
 
+long long marlin_amd_scratch_bytes(int dev, int* buffers) {
+  return (long long)scratch_bytes_held(dev, buffers);
+}
+
+long long marlin_amd_release(int dev) { return (long long)scratch_release(dev); }
+
+int marlin_amd_device_info(int dev, int* out) {
+  const hipDeviceAttribute_t what[5] = {
+      hipDeviceAttributeMultiprocessorCount, hipDeviceAttributeClockRate,
+      hipDeviceAttributeMemoryClockRate, hipDeviceAttributeMemoryBusWidth,
+      hipDeviceAttributeL2CacheSize};
+  for (int i = 0; i < 5; i++) {
+    out[i] = 0;
+    hipError_t e = hipDeviceGetAttribute(&out[i], what[i], dev);
+    if (e != hipSuccess) {
+      set_error(e, "hipDeviceGetAttribute");
+      return MARLIN_ERR_RUNTIME;
+    }
+  }
+  return MARLIN_OK;
+}
+
+int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  int tk = -1, tn = -1;
+  int rc = check_shape(1, prob_n, prob_k, -1, tk, tn);
+  if (rc != MARLIN_OK) return rc;
+  if (prob_n == 0 || prob_k == 0 || dev < 0 || dev >= kMaxDevices) return MARLIN_ERR_PROB_SHAPE;
+  const int cus = device_cus(dev);
+  if (cus <= 0) return MARLIN_ERR_RUNTIME;
+  const PlanCtx cx = {cus, kPoolPartialLimit, Force()};
+  const Plan pl = make_plan(1, prob_n, prob_k, -1, cx);
+  (void)hipGetLastError();
+  if (kind == 0) {
+    rc = launch_probe_empty(pl.grid, stream);
+  } else {
+    GemmArgs a = {};
+    a.B = B;
+    a.M = 1;
+    a.N = prob_n;
+    a.K = prob_k;
+    a.gpb = pl.sp.gpb;
+    a.wpt = pl.sp.wpt;
+    rc = launch_probe_read(a, pl.grid, stream);
+  }
+  if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "probe launch");
+  return rc;
+}
+
 const char* marlin_amd_last_error(void) { return g_last_error; }
 
-const char* marlin_amd_version(void) { return "marlin_amd 0.1 (gfx950)"; }
+const char* marlin_amd_version(void) { return "marlin_amd 0.2 (gfx950)"; }
 
 }  // extern "C"

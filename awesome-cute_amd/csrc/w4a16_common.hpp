@@ -146,12 +146,18 @@ __host__ __device__ __forceinline__ int tile_last_block(const StreamPlan& p, int
   return ((t + 1) * p.KG - 1) / p.gpb;
 }
 
-// Every workgroup owns at most two tiles that it shares with others (its
-// first and its last); a shared tile's partial sums go to slot 2b or 2b+1.
+// Partial-sum slots: two per workgroup.  In the first form a workgroup owns at
+// most two tiles that it shares with others (its first and its last), whose
+// partial sums go to slot 2b and 2b+1; in the second form it has one tile and
+// uses slot 2b only (slots 16 KiB apart measured 0.1-0.2 us faster per launch
+// than slots packed 8 KiB apart at 1-16 rows).
 __host__ __device__ __forceinline__ int partial_slot(const StreamPlan& p, int block, int t) {
+  if (p.wpt > 0) return 2 * block;
   // block touches tile t; t is its first tile unless the block starts before it
   return 2 * block + (block * p.gpb < t * p.KG ? 1 : 0);
 }
+// slots a launch of plan p may touch
+__host__ __device__ __forceinline__ int stream_slots(const StreamPlan& p) { return 2 * p.grid; }
 
 struct GemmArgs {
   const void* A;    // (M, K) fp16 row-major
@@ -161,7 +167,7 @@ struct GemmArgs {
   int M, N, K;
   int* locks;       // N/128 counters, lock_stride ints apart; zero on entry and on exit
   int lock_stride;  // >= 1; spreads the counters over separate cache lines
-  float* scratch;   // partial sums of shared tiles
+  float* scratch;   // partial sums of shared tiles (null if no tile is shared)
   int gpb;          // granules per workgroup (streaming kernel; the most, when wpt > 0)
   int wpt;          // workgroups per column tile, or 0 (see StreamPlan)
 };
@@ -180,5 +186,11 @@ int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 // counter per tile, zero again afterwards)
 // tile_rows: rows of C per workgroup, 64 or 128
 int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream);
+
+// Measurement probes (w4a16_probe.hip): an empty launch of `grid` workgroups,
+// and a plain read of the packed weights with the streaming kernel's work split
+// (a.B, a.N, a.K, a.gpb, a.wpt) and access pattern, no arithmetic.
+int launch_probe_empty(int grid, hipStream_t stream);
+int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream);
 
 }  // namespace w4a16

@@ -27,22 +27,6 @@
 // dealt out two behind every MFMA, where they cost no issue time.
 #include "w4a16_common.hpp"
 
-// Tuning builds may remap the k stage that is fetched (e.g. to a cache-hot
-// one); the library build fetches the stage it computes.
-#ifndef W4A16_PF_K
-#define W4A16_PF_K(s) (s)
-#endif
-#ifndef W4A16_PF_T0
-#define W4A16_PF_T0
-#define W4A16_PF_T1
-#define W4A16_PF_TBEGIN
-#define W4A16_PF_TEND
-#endif
-#ifndef W4A16_PF_TENTRY
-#define W4A16_PF_TENTRY
-#define W4A16_PF_TEXIT
-#endif
-
 namespace w4a16 {
 
 namespace {
@@ -78,7 +62,6 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
                                                       int ksplit) {
   extern __shared__ __attribute__((aligned(16))) char smem_all[];  // PfShape<RB>::kLdsBytes
   __shared__ int s_ticket;
-  W4A16_PF_TENTRY
   {
     // fetch every kernel argument in one round trip (the compiler would fetch
     // the pointers in a second one, just before the first load needs them)
@@ -185,27 +168,20 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     const int inv = sg < s_end ? 0 : kOobPf;
     if (GROUP)
       sreg[slot] = __builtin_amdgcn_raw_buffer_load_b64(rS, s_lane | inv,
-                                                        (W4A16_PF_K(sg) >> 1) * p.N * 2, 0);
+                                                        (sg >> 1) * p.N * 2, 0);
   };
   auto issue_a = [&](int s) {
     const int sg = s_begin + s;
     const int inv = sg < s_end ? 0 : kOobPf;
-#ifndef W4A16_PF_SKIP_A
 #pragma unroll
     for (int i = 0; i < HB; i++)
-      areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
-#endif
-#ifndef W4A16_PF_SKIP_B
+      areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, sg * 128, 0);
 #pragma unroll
     for (int i = 0; i < 2; i++)
       bcopy[i] = __builtin_amdgcn_raw_buffer_load_b128(
-          rB, b_ld | inv, (4 * W4A16_PF_K(sg) + 2 * i + (wave >> 1)) * b_row, 0);
-#endif
+          rB, b_ld | inv, (4 * sg + 2 * i + (wave >> 1)) * b_row, 0);
   };
   auto store_a = [&](int ring) {
-#ifdef W4A16_PF_SKIP_ST
-    return;
-#endif
     char* base = smem + ring * kPfStageBytes;
 #pragma unroll
     for (int i = 0; i < HB; i++)
@@ -224,18 +200,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   h8 w[2][4];  // unpacked weights of the current and the next k step
   i4 af[4];    // ring of activation operands, three ahead of the MFMAs
   i2 bw[2];    // packed weight words of the next k step (its two 16-deep rows)
-#ifdef W4A16_PF_INIT
-  for (int i = 0; i < HB; i++) areg[i] = (i4){tid, 1, 2, 3};
-  for (int i = 0; i < 4; i++) af[i] = (i4){tid, 5, 6, 7};
-  for (int i = 0; i < 2; i++) { bcopy[i] = (i4){tid, 9, 1, 2}; sreg[i] = (i2){tid, 3}; }
-  for (int i = 0; i < 2; i++) for (int j = 0; j < 4; j++) w[i][j] = __builtin_bit_cast(h8, (i4){tid, j, i, 7});
-#endif
 
   // unpack the two words of 16-column group j2 of k step (slot, h) into w[buf]
   auto dequant_pair = [&](int buf, int slot, int h, int j2) {
-#ifdef W4A16_PF_SKIP_DQ
-    return;
-#endif
     (void)h;
     h2 s2 = GROUP ? as_h2(sreg[slot][j2]) : (h2){(half_t)1.f, (half_t)1.f};
     h2 l0, h0, l1, h1, m0_, n0_, m1_, n1_;
@@ -246,16 +213,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   };
   // fetch the packed words of k step h of the slab at `stage_base`
   auto read_bw = [&](const char* stage_base, int h) {
-#ifdef W4A16_PF_SKIP_RD
-    return;
-#endif
     bw[0] = *(const i2*)(stage_base + b_rd + (2 * h) * 2048);
     bw[1] = *(const i2*)(stage_base + b_rd + (2 * h + 1) * 2048);
   };
   auto read_frag = [&](int idx, const char* step_base, int i) {
-#ifdef W4A16_PF_SKIP_RD
-    return;
-#endif
     af[idx] = *(const i4*)(step_base + a_rd + i * 256);
   };
 
@@ -319,12 +280,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
         for (int u = 0; u < kPairsPerMfma; u++) {
           const int t = (m - kFirst) * kPairsPerMfma + u;
-#ifndef W4A16_PF_SKIP_DQ
           if (t >= 0 && t < 2 * kOpsPerWord) {
             dq_op(h ^ 1, nslot, t / kOpsPerWord, 0, t % kOpsPerWord);
             dq_op(h ^ 1, nslot, t / kOpsPerWord, 1, t % kOpsPerWord);
           }
-#endif
         }
         extra(m);
         __builtin_amdgcn_sched_barrier(0);
@@ -340,9 +299,6 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     constexpr int kBegin = 4 * RB - (HB * kPerA + 2 * 2);
     const int x = m - kBegin;
     if (x < 0) return;
-#ifdef W4A16_PF_SKIP_TRAFFIC
-    return;
-#endif
     char* base = smem + ring_next * kPfStageBytes;
     const int sg = s_begin + s_next2;
     const int inv = sg < s_end ? 0 : kOobPf;
@@ -353,14 +309,14 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
         *(int*)(base + a_wr + (2 * g) * kPlane + i * 32 * 16) = areg[i][2 * g];
         *(int*)(base + a_wr + (2 * g + 1) * kPlane + i * 32 * 16) = areg[i][2 * g + 1];
       } else
-        areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, W4A16_PF_K(sg) * 128, 0);
+        areg[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, a_lane[i] | inv, sg * 128, 0);
     } else {
       const int y = x - HB * kPerA, i = y >> 1;
       if ((y & 1) == 0)
         *(i4*)(base + b_wr + i * 4096) = bcopy[i];
       else
         bcopy[i] = __builtin_amdgcn_raw_buffer_load_b128(
-            rB, b_ld | inv, (4 * W4A16_PF_K(sg) + 2 * i + (wave >> 1)) * b_row, 0);
+            rB, b_ld | inv, (4 * sg + 2 * i + (wave >> 1)) * b_row, 0);
     }
   };
 
@@ -383,7 +339,6 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // slower, up to 4 % faster depending on the schedule of the loop).
   if (kh) __builtin_amdgcn_s_setprio(1);
   int ring = 0;  // LDS slab of the stage being computed
-  W4A16_PF_TBEGIN
   for (int s = 0; s < stages; s += 2) {
 #pragma unroll
     for (int u = 0; u < 2; u++) {
@@ -402,11 +357,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       // enough; it sits mid-stage, where no wave needs the new slab yet.
       step(0, cur, cur + kPfStepBytes, cur, u, 1,
            [&](int m) { stage_traffic(m, ring_next, cs + 2); });
-      W4A16_PF_T0
-#ifndef W4A16_PF_NO_BARRIER
       __syncthreads();
-#endif
-      W4A16_PF_T1
       // step 1: the scales of this stage are spent, request those of stage cs+2
       step(1, cur + kPfStepBytes, nxt, nxt, u ^ 1, 0, [](int) {});
       issue_s(u, cs + 2);
@@ -414,7 +365,6 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     }
   }
 
-  W4A16_PF_TEND
   // ---- epilogue.  The k halves swap the row blocks they will not write
   // (half 0 keeps blocks 0..HB-1, half 1 the rest) through LDS and add; the
   // slab rings are dead by now.
@@ -530,7 +480,6 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       __builtin_nontemporal_store(v, (i4*)(C + (size_t)(m0 + m) * p.N + kPfTileN * tn + c16 * 8));
     }
   }
-  W4A16_PF_TEXIT
 }
 
 template <int RB>

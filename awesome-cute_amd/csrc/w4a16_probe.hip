@@ -1,0 +1,78 @@
+// Measurement probes: what a launch and a plain read of the packed weights cost
+// on this device, with no arithmetic, to judge the GEMM kernels against.
+//
+// probe_read_kernel walks the packed weights exactly as the streaming kernel
+// does for the same plan -- same work split, same workgroup-to-XCD order, same
+// 128-bit streaming buffer loads of 1 KiB per wave instruction, four rows per
+// granule -- keeps up to kProbeDepth granules in flight per wave, and throws
+// the data away.  probe_empty_kernel does nothing at all.
+#include "w4a16_common.hpp"
+
+namespace w4a16 {
+
+namespace {
+constexpr int kProbeDepth = 4;
+constexpr int kProbeOob = (int)0x80000000;
+}  // namespace
+
+__global__ __launch_bounds__(256) void probe_empty_kernel() {}
+
+__global__ __launch_bounds__(256) void probe_read_kernel(GemmArgs p, int* sink) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int kg = lane >> 4, nu = lane & 15;
+  const int NT = p.N / kTileN, KG = p.K / kGranuleK;
+  const int total = NT * KG;
+  const int wid = xcd_work_index((int)blockIdx.x, (int)gridDim.x);
+  int u0, u1;
+  if (p.wpt > 0) {
+    const int t = wid / p.wpt, run = wid - t * p.wpt;
+    u0 = t * KG + (run * KG) / p.wpt;
+    u1 = t * KG + ((run + 1) * KG) / p.wpt;
+    if (t >= NT) return;
+  } else {
+    u0 = wid * p.gpb;
+    u1 = min(total, u0 + p.gpb);
+  }
+  const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void*>(p.B), 0, (int)((unsigned)p.K * (unsigned)(p.N / 2)), 0x00020000);
+  const int b_row = p.N * 8;
+  const int b_lane = 64 * nu + 16 * kg;
+  i4 acc = {0, 0, 0, 0};
+  i4 buf[kProbeDepth][4];
+  auto issue = [&](int slot, int u) {
+    const bool valid = u < u1;
+    const int t = u / KG, kq = u - t * KG;
+    const int vb = b_lane | (valid ? 0 : kProbeOob);
+    const int sb = valid ? (4 * kq) * b_row + 1024 * t : 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      buf[slot][r] = __builtin_amdgcn_raw_buffer_load_b128(rB, vb, sb + r * b_row, 2);
+  };
+  int u = u0 + wave;
+#pragma unroll
+  for (int d = 0; d < kProbeDepth; d++) issue(d, u + 4 * d);
+  for (; u < u1; u += 4 * kProbeDepth) {
+#pragma unroll
+    for (int d = 0; d < kProbeDepth; d++) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc |= buf[d][r];
+      issue(d, u + 4 * (d + kProbeDepth));
+    }
+  }
+  // uniform packed nibbles never OR to this pattern: nothing is written
+  if ((acc[0] & acc[1] & acc[2] & acc[3]) == 0x12345678 && sink) sink[0] = 1;
+}
+
+int launch_probe_empty(int grid, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(256), 0, stream);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, a, (int*)nullptr);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+}  // namespace w4a16

@@ -22,12 +22,6 @@
 // flight while the current tile is reduced and written.
 #include "w4a16_common.hpp"
 
-// Optional phase timestamps for tuning builds; empty in the library build.
-#ifndef W4A16_STAMP_DECL
-#define W4A16_STAMP_DECL
-#define W4A16_STAMP(i)
-#endif
-
 namespace w4a16 {
 
 namespace {
@@ -141,7 +135,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   using Lds = StreamLds<MB, DEPTH, ONE_TILE>;
   constexpr bool kDmaA = Lds::kDmaA;
 
-  W4A16_STAMP_DECL
   {
     // Fetch every kernel argument now, in one round trip: left alone, the
     // compiler fetches the pointers only behind the early exit below, a second
@@ -339,12 +332,10 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // ---- sum the four waves; wave w ends up owning the 16-column groups
     // (j = w, h = 0/1) of every row block
     f4 res[MB][2];
-    W4A16_STAMP(3)
     // where the reduction reuses the ring's memory, the (empty) ring loads still
     // in flight must have landed before anybody writes there
     if constexpr (Lds::kAliased) __builtin_amdgcn_s_waitcnt(kWaitVm0);
     lds_barrier();
-    W4A16_STAMP(4)
     if constexpr (Lds::kAliased) {
       // room for all row blocks at once: two barriers instead of two per block
 #pragma unroll
@@ -383,7 +374,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       }
     }
 
-    W4A16_STAMP(5)
     // ---- meet the other workgroups of this tile, if any.  Partial sums are
     // written with device-scope (write-through) stores, whole 1 KiB lines per
     // wave instruction, so no cache write-back is needed: a wave waits until
@@ -416,7 +406,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
-      W4A16_STAMP(6)
       writer = (s_ticket == bl - bf);
       if (writer) {
         // Add the partials in workgroup order (deterministic).  They are fetched
@@ -465,7 +454,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       __syncthreads();  // s_ticket is reused by the next tile
     }
 
-    W4A16_STAMP(7)
     // ---- write C (fp16); per-channel mode scales the rounded result
     if (writer) {
       half_t* C = (half_t*)p.C;
@@ -505,7 +493,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       issue(d, my_tile, ikq, d < n_mine);
       ikq += 4;
     }
-    W4A16_STAMP(1)
     if constexpr (DEPTH == 2 && !kDmaA) {
       // At most two granules per wave and both are already requested: a rolled
       // loop over one copy of the compute code; the second granule moves into
@@ -513,7 +500,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 #pragma unroll 1
       for (int i = 0; i < n_mine; i++) {
         compute(0);
-        if (i == 0) { W4A16_STAMP(2) }
 #pragma unroll
         for (int r = 0; r < 4; r++) bq[0][r] = bq[1][r];
         sq[0] = sq[1];
@@ -530,7 +516,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           // the slots past the end hold zeros: skip their arithmetic (the loads
           // are still issued, so the load counter stays exact)
           if (base + d < n_mine) compute(d);
-          if (base + d == 0) { W4A16_STAMP(2) }
           issue(d, my_tile, ikq, base + d + DEPTH < n_mine);
           ikq += 4;
         }
@@ -560,7 +545,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       }
     }
 
-    W4A16_STAMP(1)
     for (int base = 0; base < n_mine; base += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; d++) {
@@ -574,7 +558,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           }
         }
         if (i < n_mine) compute(d);  // the slots past the end hold zeros
-        if (i == 0) { W4A16_STAMP(2) }
         ckq += 4;
         while (ckq >= KG) {
           ckq -= KG;
@@ -594,7 +577,6 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       clear_acc();
     }
   }
-  W4A16_STAMP(8)
 }
 
 // Ring depth of the deep variant.  Three granules in flight per wave measured

@@ -25,8 +25,17 @@ _I = ctypes.c_int
 _lib.marlin_mul.restype = _I
 _lib.marlin_mul.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P, ctypes.c_longlong, _I, _P,
                             _I, _I, _I, _I, _I, ctypes.c_char_p, _I]
-_lib.marlin_gemm.restype = _I
-_lib.marlin_gemm.argtypes = [_P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I]
+for _name in ("marlin_gemm", "marlin_cute", "marlin_official"):
+    getattr(_lib, _name).restype = _I
+    getattr(_lib, _name).argtypes = [_P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I]
+_lib.marlin_amd_scratch_bytes.restype = ctypes.c_longlong
+_lib.marlin_amd_scratch_bytes.argtypes = [_I, _P]
+_lib.marlin_amd_release.restype = ctypes.c_longlong
+_lib.marlin_amd_release.argtypes = [_I]
+_lib.marlin_amd_probe.restype = _I
+_lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _P]
+_lib.marlin_amd_device_info.restype = _I
+_lib.marlin_amd_device_info.argtypes = [_I, _P]
 _lib.marlin_amd_check.restype = _I
 _lib.marlin_amd_check.argtypes = [_I] * 6
 _lib.marlin_amd_plan.restype = _I
@@ -233,17 +242,17 @@ def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
 
 
 def force_kernel(which):
-    """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel (process-wide)."""
+    """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel (calling thread only)."""
     _lib.marlin_amd_force_kernel(int(which))
 
 
 def force_k_slices(slices):
-    """Slices of the k range per prefill tile; 0 = choose by cost (process-wide)."""
+    """Slices of the k range per prefill tile; 0 = choose by cost (calling thread only)."""
     _lib.marlin_amd_force_k_slices(int(slices))
 
 
 def force_tile_rows(rows):
-    """Rows of C per prefill workgroup (64 or 128); 0 = choose by cost (process-wide)."""
+    """Rows of C per prefill workgroup (64 or 128); 0 = choose by cost (calling thread only)."""
     _lib.marlin_amd_force_tile_rows(int(rows))
 
 
@@ -256,8 +265,52 @@ def work_order(grid):
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     """Kernel, grid and stream-K partition marlin_gemm would use."""
-    out = (ctypes.c_int * 9)()
+    out = (ctypes.c_int * 10)()
     rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
     keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
-            "k_slices", "tile_rows", "wgs_per_tile")
+            "k_slices", "tile_rows", "wgs_per_tile", "partial_kib")
     return rc, dict(zip(keys, out))
+
+
+def scratch_bytes(dev=-1):
+    """(bytes, buffers) of partial-sum scratch the library holds (no GPU touched)."""
+    n = ctypes.c_int(0)
+    return _lib.marlin_amd_scratch_bytes(dev, ctypes.byref(n)), n.value
+
+
+def release(dev=-1):
+    """Free the library's partial-sum scratch (waits for the device); bytes freed."""
+    return _lib.marlin_amd_release(dev)
+
+
+def device_info(dev=0):
+    """Compute units, shader clock (kHz), memory clock (kHz), bus width (bits), L2 bytes."""
+    out = (ctypes.c_int * 5)()
+    if _lib.marlin_amd_device_info(dev, out) != 0:
+        raise RuntimeError(_lib.marlin_amd_last_error().decode())
+    return dict(zip(("compute_units", "clock_khz", "memory_clock_khz", "bus_width_bits",
+                     "l2_bytes"), out))
+
+
+def gemm_raw(entry, A, B, C, s, workspace, groupsize, thread_k=-1, thread_n=-1, sms=-1,
+             max_par=16, stream=None):
+    """One of the 15-argument C entries (`marlin_gemm`, `marlin_cute`, `marlin_official`)
+    on tensors: returns the entry's integer code."""
+    dev = A.get_device()
+    return getattr(_lib, entry)(A.data_ptr(), B.data_ptr(), C.data_ptr(), s.data_ptr(),
+                                A.size(0), C.size(1), A.size(1), workspace.data_ptr(), groupsize,
+                                dev, _raw_stream(dev) if stream is None else stream,
+                                thread_k, thread_n, sms, max_par)
+
+
+def probe(kind, B, n, k):
+    """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
+    packed weights B with the streaming kernel's work split (marlin_amd_probe)."""
+    dev = B.get_device()
+    rc = _lib.marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev))
+    if rc != 0:
+        raise RuntimeError(f"marlin_amd_probe failed with code {rc}: {last_error()}")
+
+
+def last_error():
+    return _lib.marlin_amd_last_error().decode()

@@ -6,8 +6,14 @@ seeded inputs already resident in HBM.  Memory-bound shapes rotate over enough
 distinct weight/scale buffers to exceed the 256 MB Infinity Cache, so the
 figure is an HBM figure and not a cache figure.  The K timed steps are captured
 in one HIP graph (kernel launches only) and bracketed by HIP events on the
-launch stream, so the host's launch cost is not part of the kernel's number;
-the eager (one host call per step) rate is reported next to it.
+launch stream, so the host's launch cost is not part of the kernel's number.
+The graph is replayed until at least 50 ms of GPU time and 20 replays have been
+timed (each replay is exactly K steps; a pair of events brackets enough
+back-to-back replays to cover 200 launches; when K is smaller than the number
+of rotated weight buffers, several K-step graphs that continue the rotation
+take turns); `ms_per_step` is the median sample, the spread is reported
+beside it.  The eager (one host call per step) rate is
+reported next to it.
 
 Prints ONE JSON line: the headline workload is the decode configuration (
 M=1, N=K=4096, group 128), with `roofline` for its kernel and `cpu_baseline`
@@ -76,7 +82,47 @@ def build_inputs(torch, O, M, N, K, groupsize, nbuf, seed=0):
     return (A, B, sp), dA, dBs, dSs, dC, ws
 
 
-def time_shape(torch, marlin, O, name, steps, warmup, check=True):
+def graph_ms(torch, side, fn, steps, period):
+    """Median time (ms) of one step over replays of graphs of exactly `steps`
+    calls fn(i).  i runs on from graph to graph, so `period` distinct buffers
+    are all visited even when steps < period.  Returns (median, (min, max,
+    samples))."""
+    n_graphs = max(1, min(8, -(-period // steps)))
+    graphs = []
+    for g in range(n_graphs):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(steps):
+                fn(g * steps + i)
+        graphs.append(graph)
+    cur = torch.cuda.current_stream()
+    for g in graphs:  # untimed: uploads the graph, brings the clocks up
+        g.replay()
+    torch.cuda.synchronize()
+    # one pair of events brackets `per_sample` back-to-back replays (at least
+    # 200 launches), so that what a graph launch costs by itself weighs little
+    per_sample = max(1, -(-200 // steps))
+    times, total, r = [], 0.0, 0
+    while (total < 50.0 or r < 20 or len(times) < 15) and r < 20000:
+        batch = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(cur)
+            for _ in range(per_sample):
+                graphs[r % n_graphs].replay()
+                r += 1
+            e1.record(cur)
+            batch.append((e0, e1))
+        torch.cuda.synchronize()
+        for e0, e1 in batch:
+            t = e0.elapsed_time(e1)
+            times.append(t / (steps * per_sample))
+            total += t
+    times.sort()
+    return times[len(times) // 2], (times[0], times[-1], len(times))
+
+
+def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=False):
     M, N, K, g, bound = SHAPES[name]
     weight_bytes = K * N // 2
     nbuf = max(2, -(-2 * MALL_BYTES // weight_bytes)) if bound == "hbm" else 2
@@ -113,31 +159,30 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True):
         eager_ms = (time.perf_counter() - t0) * 1e3 / steps
         eager_dev_ms = e0.elapsed_time(e1) / steps
 
-    def graph_ms(fn):
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            for i in range(steps):
-                fn(i)
-        for _ in range(2):
-            graph.replay()
-        torch.cuda.synchronize()
-        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        cur = torch.cuda.current_stream()
-        g0.record(cur)
-        graph.replay()
-        g1.record(cur)
-        torch.cuda.synchronize()
-        return g0.elapsed_time(g1) / steps
-
-    ms = graph_ms(call)
+    ms, spread = graph_ms(torch, side, call, steps, nbuf)
     # the same launches over one weight buffer, which then stays in the 256 MB
     # Infinity Cache / L2: the figure kernel timings on other hardware usually are
-    resident_ms = graph_ms(lambda i: call(0)) if bound == "hbm" and nbuf > 1 else None
+    resident_ms = (graph_ms(torch, side, lambda i: call(0), steps, 1)[0]
+                   if bound == "hbm" and nbuf > 1 else None)
+    floor = None
+    if with_floor:
+        # what the launch alone and the weight stream alone cost, measured the same way
+        e_ms, _ = graph_ms(torch, side, lambda i: marlin.probe(0, dBs[0], N, K), steps, 1)
+        r_ms, r_spread = graph_ms(torch, side, lambda i: marlin.probe(1, dBs[i % nbuf], N, K),
+                                  steps, nbuf)
+        floor = {"empty_kernel_us": e_ms * 1e3, "read_kernel_us": r_ms * 1e3,
+                 "read_kernel_spread_us": [x * 1e3 for x in r_spread[:2]],
+                 "read_GBps": weight_bytes / (r_ms * 1e-3) / 1e9,
+                 "what": "same grid and work split as the GEMM launch; read kernel = the packed "
+                         "weights through the streaming kernel's 128-bit loads, no arithmetic, "
+                         "nothing written; same buffer rotation and graph timing"}
 
     flops = 2.0 * M * N * K
     res = {
         "name": name, "M": M, "N": N, "K": K, "groupsize": g,
         "ms_per_step": ms, "us_per_launch": ms * 1e3,
+        "us_per_launch_min_max": [spread[0] * 1e3, spread[1] * 1e3], "graph_replays": spread[2],
+        "stream_floor": floor,
         "eager_ms_per_step": eager_ms, "eager_device_ms_per_step": eager_dev_ms,
         "weight_GBps": weight_bytes / (ms * 1e-3) / 1e9,
         "tflops": flops / (ms * 1e-3) / 1e12,
@@ -211,7 +256,7 @@ def main():
 
     if args.shape == "headline":
         main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128",
-                                        "decode_large"]
+                                        "large_chan", "decode_large"]
     else:
         main_name, others = args.shape, []
 
@@ -231,15 +276,18 @@ def main():
         del src, dst
 
     prop = torch.cuda.get_device_properties(0)
+    info = marlin.device_info(0)  # from the HIP runtime, through the C ABI
     # cross-check of the published matrix peak: CUs x 4 SIMDs x 1024 fp16 flop per clock x clock
-    clock_khz = getattr(prop, "clock_rate", None)  # not exposed by every torch build
+    clock_hz = info["clock_khz"] * 1e3
     peaks = {"hbm_GBps": HBM_PEAK_GBPS, "mfma_fp16_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
-             "device": prop.name, "compute_units": prop.multi_processor_count,
-             "clock_MHz": None if clock_khz is None else clock_khz / 1e3,
-             "mfma_fp16_TFLOPs_at_2400MHz": prop.multi_processor_count * 4 * 1024 * 2.4e9 / 1e12,
-             "mfma_fp16_TFLOPs_from_clock": None if clock_khz is None else
-                 prop.multi_processor_count * 4 * 1024 * clock_khz * 1e3 / 1e12}
-    head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup)
+             "device": prop.name, "compute_units": info["compute_units"],
+             "clock_MHz": info["clock_khz"] / 1e3,
+             "mfma_fp16_TFLOPs_from_clock": info["compute_units"] * 4 * 1024 * clock_hz / 1e12,
+             "memory_clock_MHz": info["memory_clock_khz"] / 1e3,
+             "memory_bus_bits": info["bus_width_bits"],
+             # HBM3E transfers twice per memory clock
+             "hbm_GBps_from_clock": info["memory_clock_khz"] * 1e3 * 2 * info["bus_width_bits"] / 8 / 1e9}
+    head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup, with_floor=True)
     shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup) for n in others]
 
     M, N, K, g, bound = SHAPES[main_name]
@@ -253,7 +301,11 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"{main_name}: M={M} N={N} K={K} groupsize={g} W4A16 GEMM",
                    "weight_buffers_rotated": head["weight_buffers_rotated"],
-                   "timing": "K launches in one HIP graph, HIP events on the launch stream"},
+                   "timing": "K launches in one HIP graph, replayed for >= 50 ms and >= 20 "
+                             "replays, HIP events around every >= 200 launches, median sample"},
+        "us_per_launch_min_max": head["us_per_launch_min_max"],
+        "graph_replays": head["graph_replays"],
+        "stream_floor": head["stream_floor"],
         "tflops": head["tflops"], "weight_GBps": head["weight_GBps"],
         "cache_resident_us_per_launch": head["cache_resident_us_per_launch"],
         "peaks": peaks,

@@ -44,8 +44,15 @@ extern "C" {
  *       ((128,128) up to 16 rows, else (64,256)).  They are validated exactly
  *       as the reference validates them but do not select the kernel.
  *   sms        number of workgroups of the streaming kernel, -1 = automatic
- *   max_par    only sizes the workspace contract
+ *   max_par    at least 1 (else MARLIN_ERR_WORKSPACE); sizes the workspace
+ *       contract, and the tile counters sit min(max_par, 16) ints apart in it
  * Not re-entrant over the same workspace or the same C concurrently.
+ * Partial sums of output tiles that several workgroups share live in a
+ * library-owned buffer per (device, stream), sized by the call's plan and
+ * grown on demand (hipMalloc on the first call that needs more; 64 KiB of tile
+ * counters + whole MiB of partial sums, 4 MiB for N = K = 4096 at one row).  A call that
+ * would have to allocate while `stream` is being captured into a graph returns
+ * MARLIN_ERR_RUNTIME: run the call once on that stream before the capture.
  */
 int marlin_gemm(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
                 int prob_k, void *workspace, int groupsize, int dev, void *stream, int thread_k,
@@ -65,7 +72,7 @@ int marlin_official(const void *A, const void *B, void *C, void *s, int prob_m, 
  * (marlin_gemm.cpp:19-56) on plain sizes: derives groupsize from the number
  * of scale rows (1 row = per-channel), rejects k not divisible into the
  * groups (MARLIN_ERR_GROUPS) and a workspace shorter than
- * prob_n/128*max_par entries (MARLIN_ERR_WORKSPACE), calls marlin_gemm and,
+ * prob_n/128*max(max_par,1) entries (MARLIN_ERR_WORKSPACE), calls marlin_gemm and,
  * on any error, writes the reference's message text into err (if non-null).
  */
 int marlin_mul(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
@@ -87,7 +94,8 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * workgroup (prefill; 0 for the streaming kernel), out[8] = workgroups per
  * column tile when the streaming kernel cuts every tile into that many runs
  * (then out[2] is the longest run), 0 when it cuts the tile-major sequence of
- * granules into equal runs of out[2].  `out` holds 9 ints.
+ * granules into equal runs of out[2]; out[9] = KiB of partial sums the launch
+ * exchanges through the library's scratch (0 = none).  `out` holds 10 ints.
  * Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
@@ -104,25 +112,60 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
 void marlin_amd_work_order(int grid, int *out);
 
 /*
- * Which kernel marlin_gemm uses, process-wide: 0 = choose by cost (default),
- * 1 = the streaming kernel, 64 rows per launch, 2 = the prefill kernel (needs
- * prob_n % 256 == 0, else the streaming kernel is used).  No reference
- * counterpart; for tests and tools.
+ * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
+ * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
+ * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is
+ * used).  Like the two overrides below it is kept per host thread, so it never
+ * changes what other threads' calls do.  No reference counterpart; for tests
+ * and tools.
  */
 void marlin_amd_force_kernel(int which);
 
 /*
- * Slices of the k range per tile of the prefill kernel, process-wide: 0 =
- * choose by cost (default), n = n slices where the problem allows (each slice
+ * Slices of the k range per tile of the prefill kernel, for the calling
+ * thread: 0 = choose by cost (default), n = n slices where the problem allows (each slice
  * at least 256 deep).  No reference counterpart; for tests and tools.
  */
 void marlin_amd_force_k_slices(int slices);
 
 /*
- * Rows of C per workgroup of the prefill kernel, process-wide: 0 = choose by
- * cost (default), 64 or 128.  No reference counterpart; for tests and tools.
+ * Rows of C per workgroup of the prefill kernel, for the calling thread: 0 =
+ * choose by cost (default), 64 or 128.  No reference counterpart; for tests and tools.
  */
 void marlin_amd_force_tile_rows(int rows);
+
+/*
+ * Device memory the library holds for partial sums on device dev (all devices
+ * if dev < 0): returns the bytes, *buffers (if non-null) the number of
+ * (device, stream) buffers.  Touches no GPU.  No reference counterpart.
+ */
+long long marlin_amd_scratch_bytes(int dev, int *buffers);
+
+/*
+ * Frees the partial-sum buffers of device dev (all devices if dev < 0) after
+ * waiting for the device's work; returns the bytes freed.  Graphs captured
+ * earlier name the freed buffers and must not be replayed afterwards.  The
+ * next call that needs scratch allocates again.  No reference counterpart (the
+ * reference keeps its partial sums in C).
+ */
+long long marlin_amd_release(int dev);
+
+/*
+ * out[0..4] = compute units, shader clock (kHz), memory clock (kHz), memory
+ * bus width (bits), L2 size (bytes) of device dev, as the HIP runtime reports
+ * them.  Returns MARLIN_OK or MARLIN_ERR_RUNTIME.
+ */
+int marlin_amd_device_info(int dev, int *out);
+
+/*
+ * Measurement probes on `stream` of the current device `dev`, with the grid
+ * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
+ * launch costs), kind 1 = a kernel that reads the packed weights B
+ * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
+ * 128-bit loads and does nothing with them (what the weight stream alone
+ * costs).  Nothing is written.  No reference counterpart; for benchmarks.
+ */
+int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
 
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char *marlin_amd_last_error(void);

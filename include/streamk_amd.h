@@ -24,10 +24,12 @@ extern "C" {
  * A: m x k fp16, row-major.  B: n x k fp16, row-major (the k x n column-major
  * operand of gemm_streamk.cu:29).  C: m x n fp16, row-major, written once.
  * fp32 accumulation.  m is arbitrary; n % 256 == 0 and k % 64 == 0.
- * Partial sums of the stream-K tiles live in a library-owned buffer (64 MiB +
- * 1 KiB of counters per (device, stream), allocated on the first call on a
- * stream and kept): calls on one stream may follow each other freely, calls
- * that overlap must use different streams. */
+ * Partial sums of the stream-K tiles live in the library-owned buffer of this
+ * (device, stream) that marlin_gemm uses too (include/marlin_amd.h): sized by
+ * the launch (256 KiB per slice of a stream-K tile), grown on demand, none for
+ * launches without stream-K tiles.  Calls on one stream may follow each other
+ * freely, calls that overlap must use different streams; a call that would have
+ * to allocate under graph capture returns STREAMK_ERR_RUNTIME. */
 int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, int dev,
                     void* hip_stream);
 
@@ -45,6 +47,10 @@ int streamk_amd_plan(int m, int n, int k, int cus, int* out);
 /* out[0], out[1] = row and column tile of tile number `tile` (0 <= tile <
  * tiles_m * tiles_n); for tests of the numbering */
 void streamk_amd_tile_coord(int tile, int tiles_m, int tiles_n, int* out);
+
+/* same as marlin_amd_release (include/marlin_amd.h): frees the partial-sum
+ * buffers of device dev (all if dev < 0), returns the bytes freed */
+long long streamk_amd_release(int dev);
 
 /* text of the last STREAMK_ERR_RUNTIME on this thread */
 const char* streamk_amd_last_error(void);

@@ -113,10 +113,15 @@ void w4a16_gemm_ref_f64(const uint16_t *A, const int32_t *B,
  * w: K x N fp16 bits.  Outputs q (K x N, [0,15]), s (G x N fp16 bits) and
  * ref (K x N fp16 bits, the fake-quantised weight).  s = max|w| * (2/15) per
  * group and column, q = clamp(round_half_even(w / s) + 8, 0, 15).
- * PARITY UNPINNED for the intermediate roundings of `s *= 2/15` and `w / s`
- * (the reference evaluates them with torch half kernels on a CUDA device,
- * which cannot be run here); pinned only by the invariants
- * |ref - w| <= s/2 inside the clamp range and q == 15 at the group maximum. */
+ * Pinned by tests/test_host.py (test_quantize_matches_oracle_quantiser): q, s and ref
+ * equal, bit for bit, what the reference's own sequence of torch operations
+ * (marlin_test.py:18-40: abs/amax, `s *= 2/15`, `w / s`, round, +8, clamp,
+ * `(q - 8).half() * s`) gives when torch's CPU half kernels evaluate it -- an
+ * independent library evaluation that a double rounding or a wrong tie rule
+ * fails -- plus the invariants |ref - w| <= s/2 inside the clamp range and
+ * q == 15 at the group maximum.  Residual: the reference runs those operations
+ * with torch's CUDA half kernels, which cannot be run here; IEEE half
+ * arithmetic leaves them no freedom in the results. */
 void gen_quant4_ref(const uint16_t *w, int K, int N, int groupsize,
                     uint8_t *q, uint16_t *s, uint16_t *ref);
 

@@ -35,6 +35,8 @@ def test_library_exports_every_declared_symbol(marlin):
             "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_force_kernel",
             "marlin_amd_force_k_slices", "marlin_amd_force_tile_rows",
             "marlin_amd_last_error",
+            "marlin_amd_scratch_bytes", "marlin_amd_release", "marlin_amd_device_info",
+            "marlin_amd_probe",
             "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
     for n in set(names):
@@ -345,3 +347,80 @@ def test_profiling_gen_quant4_on_cpu(marlin, groupsize):
     gs = k if groupsize == -1 else groupsize
     want = (q.astype(np.float32) - 8).astype(np.float16) * np.repeat(s, gs, axis=0)
     assert np.array_equal(want.view(np.uint16), ref.numpy().view(np.uint16))
+
+
+def test_scratch_accounting_and_plan_sizes_without_gpu(marlin):
+    """Nothing is held before any GEMM ran; the plan reports what a launch would
+    exchange through the scratch: two 8 KiB slots per workgroup and row block
+    for the streaming kernel when column tiles are shared, tile bytes per k
+    slice for the prefill kernel, nothing otherwise."""
+    assert marlin.scratch_bytes() == (0, 0)
+    assert marlin.release() == 0
+    rc, p = marlin.plan(1, 4096, 4096, 128)
+    assert rc == 0 and p["wgs_per_tile"] == 8 and p["grid"] == 256 and p["partial_kib"] == 2 * 256 * 8
+    rc, p = marlin.plan(64, 4096, 4096, 128, sms=100)  # forced uniform runs, four row blocks
+    assert p["kernel"] == 1 and p["wgs_per_tile"] == 0
+    assert p["partial_kib"] == 2 * p["grid"] * 4 * 8
+    rc, p = marlin.plan(16, 256 * 128, 1024, 128, 128, 128)  # one whole tile per workgroup
+    assert p["kernel"] == 1 and p["partial_kib"] == 0
+    rc, p = marlin.plan(2048, 4096, 4096, 128)
+    assert p["kernel"] == 2 and p["k_slices"] == 1 and p["partial_kib"] == 0
+    rc, p = marlin.plan(256, 4096, 4096, 128)
+    assert p["kernel"] == 2 and p["k_slices"] > 1
+    assert p["partial_kib"] == p["grid"] * p["tile_rows"] * 256 * 4 // 1024
+
+
+def test_streaming_grid_stays_within_the_slot_limit(marlin):
+    """However many compute units a device reports, the streaming launch has at
+    most 1024 workgroups (the bound its partial-sum slots are sized for)."""
+    for cus in (256, 1000, 2000, 5000):
+        for (m, n, k) in [(16, 4096, 4096), (1, 28672, 8192), (64, 32768, 4096)]:
+            marlin.force_kernel(1)
+            try:
+                rc, p = marlin.plan(m, n, k, 128, cus=cus)
+            finally:
+                marlin.force_kernel(0)
+            assert rc == 0 and p["grid"] <= 1024, (cus, m, n, k, p)
+            _partition(p)
+
+
+def test_planner_overrides_are_per_thread(marlin):
+    """force_kernel and friends change the plans of the calling thread only."""
+    import threading
+    seen = {}
+    marlin.force_kernel(1)
+    try:
+        def other():
+            seen["other"] = marlin.plan(2048, 4096, 4096, 128)[1]["kernel"]
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        seen["mine"] = marlin.plan(2048, 4096, 4096, 128)[1]["kernel"]
+    finally:
+        marlin.force_kernel(0)
+    assert seen == {"other": 2, "mine": 1}
+
+
+def test_max_par_below_one(marlin):
+    """max_par < 1 cannot size the tile counters: marlin_gemm refuses it, and the
+    binding asks for one counter per tile at least (the reference's comparison,
+    marlin_gemm.cpp:29-31, would let an empty workspace through)."""
+    err = ctypes.create_string_buffer(256)
+    f = marlin._lib.marlin_mul
+    rc = f(None, None, None, None, 16, 256, 128, 1, None, 0, 0, None, -1, -1, -1, 0, 1, err, 256)
+    assert rc == 5 and b"workspace must be of size at least 2" in err.value
+    g = marlin._lib.marlin_gemm
+    assert g(None, None, None, None, 16, 256, 128, None, -1, 0, None, -1, -1, -1, 0) == 5
+    assert g(None, None, None, None, 16, 256, 128, None, -1, 0, None, -1, -1, -1, -3) == 5
+
+
+def test_marlin_lib_module_signature(marlin):
+    """The module the reference imports as marlin_lib (marlin.py:5-8) with the
+    pybind defaults of marlin_gemm.cpp:58-60."""
+    import inspect
+    import marlin_lib
+    sig = inspect.signature(marlin_lib.mul)
+    assert list(sig.parameters) == ["A", "B", "C", "s", "workspace", "thread_k", "thread_n", "sms",
+                                    "max_par", "cute_version"]
+    d = {k: v.default for k, v in sig.parameters.items() if v.default is not inspect.Parameter.empty}
+    assert d == {"thread_k": -1, "thread_n": -1, "sms": -1, "max_par": 8, "cute_version": True}
