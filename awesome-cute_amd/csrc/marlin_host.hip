@@ -17,6 +17,14 @@
 #include "scratch_pool.hpp"
 #include "w4a16_common.hpp"
 
+// Scratch for partial sums and tile counters that marlin_gemm_static uses in
+// place of the pool's allocations: a fixed array in device memory, one copy per
+// GPU, addressed through the pointer hipGetSymbolAddress returns for the
+// current device (the name itself is not a device address in host code).
+constexpr size_t kStaticPartialBytes = (size_t)32 << 20;
+constexpr size_t kStaticScratchBytes = w4a16::kCounterBytes + kStaticPartialBytes;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 using namespace w4a16;
@@ -30,15 +38,22 @@ void set_error(hipError_t e, const char* what) {
   snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
 }
 
+// A fill kernel rather than a memset, so that it may be recorded into a graph.
+__global__ void scratch_clear_kernel(int* p, int count) {
+  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i < count) p[i] = 0;
+}
+
 struct DeviceState {
   int cus = 0;
   bool configured = false;          // kernels' LDS limits raised on this device
+  unsigned char* static_scratch = nullptr;  // this device's copy of `scratch`
 };
 std::mutex g_mu;
 DeviceState g_dev[kMaxDevices];
 
 // What the planner may assume about the partial-sum buffer: the pool grows up
-// to this much for one call.
+// to this much for one call; the fixed array of marlin_gemm_static is smaller.
 constexpr size_t kPoolPartialLimit = (size_t)64 << 20;
 
 // With `dev` current: raise the dynamic-LDS limit of the kernels that need it.
@@ -364,9 +379,35 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
   return rc;
 }
 
+// With `dev` current: this device's copy of the fixed scratch array, its
+// counters cleared once (on `stream`, by a kernel, so that a first call under
+// capture records the clearing like any other node).
+unsigned char* static_scratch_for(int dev, hipStream_t stream) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  DeviceState& d = g_dev[dev];
+  if (d.static_scratch) return d.static_scratch;
+  void* ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) {
+    set_error(e, "hipGetSymbolAddress(scratch)");
+    return nullptr;
+  }
+  hipLaunchKernelGGL(scratch_clear_kernel, dim3(kMaxCounters / 256), dim3(256), 0, stream,
+                     (int*)ptr, kMaxCounters);
+  e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error(e, "scratch_clear_kernel");
+    return nullptr;
+  }
+  d.static_scratch = (unsigned char*)ptr;
+  return d.static_scratch;
+}
+
+// use_static: marlin_gemm_static -- the fixed array instead of the pool, a
+// plan made for its size, and no allocation on any path.
 int run(const void* A, const void* B, void* C, const void* s, int m, int n, int k,
         void* workspace, int groupsize, int dev, hipStream_t stream, int thread_k, int thread_n,
-        int sms, int max_par) {
+        int sms, int max_par, bool use_static) {
   int rc = check_shape(m, n, k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || m == 0 || n == 0 || k == 0) return rc;
   if (max_par < 1) {
@@ -398,11 +439,26 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   const int cus = device_cus(dev);
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0 && configure_device(dev)) {
-    const PlanCtx cx = {cus, kPoolPartialLimit, t_force};
+    const PlanCtx cx = {cus, use_static ? kStaticPartialBytes : kPoolPartialLimit, t_force};
     const Plan pl = make_plan(m, n, k, sms, cx);
     ScratchView view = {nullptr, nullptr};
     bool ok = true;
-    if (pl.partial_bytes > 0) {
+    if (use_static) {
+      if (pl.partial_bytes > kStaticPartialBytes) {
+        snprintf(g_last_error, sizeof(g_last_error),
+                 "marlin_gemm_static: this call (m=%d n=%d k=%d sms=%d) needs %zu bytes of "
+                 "partial sums, the fixed scratch holds %zu: use marlin_gemm",
+                 m, n, k, sms, pl.partial_bytes, kStaticPartialBytes);
+        ok = false;
+      } else if (pl.partial_bytes > 0) {
+        unsigned char* base = static_scratch_for(dev, stream);
+        ok = base != nullptr;
+        if (ok) {
+          view.counters = (int*)base;
+          view.partials = (float*)(base + kCounterBytes);
+        }
+      }
+    } else if (pl.partial_bytes > 0) {
       ok = scratch_acquire(dev, stream, pl.partial_bytes, &view, g_last_error,
                            sizeof(g_last_error));
     }
@@ -421,7 +477,7 @@ int marlin_gemm(const void* A, const void* B, void* C, const void* s, int prob_m
                 int prob_k, void* workspace, int groupsize, int dev, void* stream, int thread_k,
                 int thread_n, int sms, int max_par) {
   return run(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, (hipStream_t)stream,
-             thread_k, thread_n, sms, max_par);
+             thread_k, thread_n, sms, max_par, false);
 }
 
 int marlin_cute(const void* A, const void* B, void* C, void* s, int prob_m, int prob_n,
@@ -437,6 +493,15 @@ int marlin_official(const void* A, const void* B, void* C, void* s, int prob_m, 
   return marlin_gemm(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream,
                      thread_k, thread_n, sms, max_par);
 }
+
+int marlin_gemm_static(const void* A, const void* B, void* C, const void* s, int prob_m,
+                       int prob_n, int prob_k, void* workspace, int groupsize, int dev,
+                       void* stream, int thread_k, int thread_n, int sms, int max_par) {
+  return run(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, (hipStream_t)stream,
+             thread_k, thread_n, sms, max_par, true);
+}
+
+long long marlin_gemm_static_capacity(void) { return (long long)kStaticPartialBytes; }
 
 int marlin_mul(const void* A, const void* B, void* C, const void* s, int prob_m, int prob_n,
                int prob_k, int s_rows, void* workspace, long long workspace_numel, int dev,

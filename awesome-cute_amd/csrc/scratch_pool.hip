@@ -77,7 +77,7 @@ bool scratch_acquire(int dev, hipStream_t stream, size_t partial_bytes, ScratchV
         snprintf(err, err_len,
                  "the stream is being captured and this call needs %zu bytes of scratch that "
                  "are not allocated yet: run the same call once on this stream before the "
-                 "capture",
+                 "capture, or use marlin_gemm_static",
                  partial_bytes + kCounterBytes);
       return false;
     }

@@ -25,9 +25,10 @@ _I = ctypes.c_int
 _lib.marlin_mul.restype = _I
 _lib.marlin_mul.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _P, ctypes.c_longlong, _I, _P,
                             _I, _I, _I, _I, _I, ctypes.c_char_p, _I]
-for _name in ("marlin_gemm", "marlin_cute", "marlin_official"):
+for _name in ("marlin_gemm", "marlin_cute", "marlin_official", "marlin_gemm_static"):
     getattr(_lib, _name).restype = _I
     getattr(_lib, _name).argtypes = [_P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I]
+_lib.marlin_gemm_static_capacity.restype = ctypes.c_longlong
 _lib.marlin_amd_scratch_bytes.restype = ctypes.c_longlong
 _lib.marlin_amd_scratch_bytes.argtypes = [_I, _P]
 _lib.marlin_amd_release.restype = ctypes.c_longlong
@@ -294,8 +295,8 @@ def device_info(dev=0):
 
 def gemm_raw(entry, A, B, C, s, workspace, groupsize, thread_k=-1, thread_n=-1, sms=-1,
              max_par=16, stream=None):
-    """One of the 15-argument C entries (`marlin_gemm`, `marlin_cute`, `marlin_official`)
-    on tensors: returns the entry's integer code."""
+    """One of the 15-argument C entries (`marlin_gemm`, `marlin_cute`, `marlin_official`,
+    `marlin_gemm_static`) on tensors: returns the entry's integer code."""
     dev = A.get_device()
     return getattr(_lib, entry)(A.data_ptr(), B.data_ptr(), C.data_ptr(), s.data_ptr(),
                                 A.size(0), C.size(1), A.size(1), workspace.data_ptr(), groupsize,

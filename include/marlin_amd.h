@@ -52,7 +52,8 @@ extern "C" {
  * grown on demand (hipMalloc on the first call that needs more; 64 KiB of tile
  * counters + whole MiB of partial sums, 4 MiB for N = K = 4096 at one row).  A call that
  * would have to allocate while `stream` is being captured into a graph returns
- * MARLIN_ERR_RUNTIME: run the call once on that stream before the capture.
+ * MARLIN_ERR_RUNTIME: run the call once on that stream before the capture, or
+ * use marlin_gemm_static.
  */
 int marlin_gemm(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
                 int prob_k, void *workspace, int groupsize, int dev, void *stream, int thread_k,
@@ -66,6 +67,29 @@ int marlin_cute(const void *A, const void *B, void *C, void *s, int prob_m, int 
 int marlin_official(const void *A, const void *B, void *C, void *s, int prob_m, int prob_n,
                     int prob_k, void *workspace, int groupsize, int dev, void *stream,
                     int thread_k, int thread_n, int sms, int max_par);
+
+/*
+ * marlin_gemm for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  Same arguments, same kernels and same results
+ * as marlin_gemm for the same plan, but partial sums and tile counters use a
+ * fixed array inside the library's device image (32 MiB + 64 KiB, held by
+ * every GPU the library runs on until the process ends) and the call never
+ * calls hipMalloc, hipFree or any allocating routine.  The plan is made for
+ * that size (fewer k slices where they would not fit); a call whose partial
+ * sums still exceed marlin_gemm_static_capacity() bytes (only an explicit
+ * `sms` above the device's compute units with more than 16 rows can) returns
+ * MARLIN_ERR_RUNTIME with a message.  All calls on one GPU share the array:
+ * calls that may overlap in time on one GPU (different streams, or graph
+ * branches) race on it and must use marlin_gemm instead.  The first call on a
+ * device looks the array's address up and clears its counters with a kernel
+ * on `stream`.
+ */
+int marlin_gemm_static(const void *A, const void *B, void *C, const void *s, int prob_m,
+                       int prob_n, int prob_k, void *workspace, int groupsize, int dev,
+                       void *stream, int thread_k, int thread_n, int sms, int max_par);
+/* bytes of partial sums the fixed array of marlin_gemm_static holds */
+long long marlin_gemm_static_capacity(void);
 
 /*
  * The checks of the reference's tensor-level binding `mul`

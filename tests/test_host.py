@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(marlin):
     assert {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul", "marlin_amd_check",
             "marlin_amd_plan", "marlin_amd_work_order", "marlin_amd_force_kernel",
             "marlin_amd_force_k_slices", "marlin_amd_force_tile_rows",
-            "marlin_amd_last_error",
+            "marlin_amd_last_error", "marlin_gemm_static", "marlin_gemm_static_capacity",
             "marlin_amd_scratch_bytes", "marlin_amd_release", "marlin_amd_device_info",
             "marlin_amd_probe",
             "marlin_amd_version"} <= set(names)
@@ -368,6 +368,7 @@ def test_scratch_accounting_and_plan_sizes_without_gpu(marlin):
     rc, p = marlin.plan(256, 4096, 4096, 128)
     assert p["kernel"] == 2 and p["k_slices"] > 1
     assert p["partial_kib"] == p["grid"] * p["tile_rows"] * 256 * 4 // 1024
+    assert marlin._lib.marlin_gemm_static_capacity() == 32 << 20
 
 
 def test_streaming_grid_stays_within_the_slot_limit(marlin):

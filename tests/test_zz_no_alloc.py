@@ -1,0 +1,135 @@
+"""GPU test of marlin_gemm_static, the entry point that allocates nothing: its
+partial sums and tile counters live in a fixed array inside the library's
+device image.  Called through the C ABI and compared, bit for bit, with
+marlin_gemm (the same plan gives the same summation order), on two calls in a
+row, the second with a smaller input; then on shapes that exercise every kind
+of exchange (shared column tiles, straddling runs, prefill k slices), the
+oracle's tolerance, the size limit's error and a HIP graph of it.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import _oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
+
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    import marlin
+    assert torch.cuda.is_available()
+    return torch, marlin
+
+
+def both(env, M, N, K, g, seed, sms=-1):
+    """marlin_gemm_static and marlin_gemm on the same device buffers."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    A, q, s, B, sp = O.make_problem(M, N, K, g, seed)
+    dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+    outs = []
+    for entry in ("marlin_gemm_static", "marlin_gemm"):
+        dC = torch.full((M, N), 3.0, dtype=torch.half, device=dev)
+        ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+        torch.cuda.synchronize()
+        print(f"  {entry} M={M} N={N} K={K} g={g} sms={sms}", flush=True)
+        rc = marlin.gemm_raw(entry, dA, dB, dC, ds, ws, g, sms=sms)
+        assert rc == 0, marlin.last_error()
+        torch.cuda.synchronize()
+        assert not ws.any().item()
+        outs.append(dC.cpu().numpy())
+    return (A, B, sp), outs[0], outs[1]
+
+
+def test_two_calls_in_a_row_second_smaller(env):
+    torch, marlin = env
+    before = marlin.scratch_bytes()
+    # both exchange partial sums through the scratch: 8 workgroups per column tile
+    (A, B, sp), c_static, c_pool = both(env, 16, 4096, 4096, 128, seed=1)
+    assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
+    r = O.compare(c_static, O.gemm(A, B, sp, 4096, 128))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+    (A, B, sp), c_static, c_pool = both(env, 3, 1024, 2048, 128, seed=2)
+    assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
+    r = O.compare(c_static, O.gemm(A, B, sp, 1024, 128))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+    # the static entry itself left the pool alone (marlin_gemm added one buffer at most)
+    after = marlin.scratch_bytes()
+    assert after[1] <= before[1] + 1
+
+
+@pytest.mark.parametrize("M,N,K,g,sms", [
+    (1, 4096, 4096, 128, -1),      # decode: every tile shared by 8 workgroups
+    (16, 1280, 1152, -1, 7),       # runs that straddle tile boundaries
+    (48, 768, 2048, 128, 100),     # LDS-ring variant, shared tiles
+    (64, 4096, 4096, 128, -1),
+    (256, 4096, 4096, 128, -1),    # prefill kernel, 64-row tiles in k slices
+    (1024, 4096, 4096, -1, -1),    # prefill kernel, 128-row tiles in 2 slices: 32 MiB, the limit
+    (2048, 1024, 1024, 128, -1),   # no exchange at all
+])
+def test_static_matches_pool_entry(env, M, N, K, g, sms):
+    torch, marlin = env
+    (A, B, sp), c_static, c_pool = both(env, M, N, K, g, seed=M + N, sms=sms)
+    assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
+    rows = slice(0, min(M, 8))
+    r = O.compare(c_static[rows], O.gemm(A[rows], B, sp, N, g))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+
+
+def test_rejects_what_does_not_fit(env):
+    """Only an explicit grid hint above the device's compute units with more than
+    16 rows needs more than the fixed 32 MiB: a clear error, nothing launched."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    assert marlin._lib.marlin_gemm_static_capacity() == 32 << 20
+    M, N, K = 64, 4096, 8192
+    A, q, s, B, sp = O.make_problem(M, N, K, 128, 9)
+    dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+    dC = torch.full((M, N), 3.0, dtype=torch.half, device=dev)
+    ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+    marlin.force_kernel(1)
+    try:
+        rc = marlin.gemm_raw("marlin_gemm_static", dA, dB, dC, ds, ws, 128, sms=1000)
+    finally:
+        marlin.force_kernel(0)
+    assert rc == 3 and "fixed scratch holds 33554432" in marlin.last_error()
+    torch.cuda.synchronize()
+    assert (dC == 3.0).all().item() and not ws.any().item()
+
+
+def test_static_entry_in_a_graph(env):
+    """Captured without a warm-up call on the capture stream (nothing to allocate), replayed
+    several times with eager launches in between: every replay gives the eager result."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    M, N, K, g = 4, 4096, 4096, 128
+    A, q, s, B, sp = O.make_problem(M, N, K, g, 12)
+    dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+    want = torch.zeros((M, N), dtype=torch.half, device=dev)
+    ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+    assert marlin.gemm_raw("marlin_gemm_static", dA, dB, want, ds, ws, g) == 0
+    torch.cuda.synchronize()
+    fresh = torch.cuda.Stream()
+    dC = torch.zeros_like(want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=fresh):
+        rc = marlin.gemm_raw("marlin_gemm_static", dA, dB, dC, ds, ws, g)
+    assert rc == 0, marlin.last_error()
+    for _ in range(4):
+        dC.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dC, want) and not ws.any().item()
+        other = torch.zeros((16, 4096), dtype=torch.half, device=dev)
+        dA16 = torch.randn((16, K), dtype=torch.half, device=dev)
+        assert marlin.gemm_raw("marlin_gemm_static", dA16, dB, other, ds, ws, g) == 0
+        torch.cuda.synchronize()
