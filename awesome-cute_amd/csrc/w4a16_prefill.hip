@@ -49,6 +49,8 @@ struct PfShape {
   // the epilogue reuses the rings: 8 waves x RB/2 row blocks x 4 KiB of fp32
   // to swap, then the fp16 tile with padded rows
   static_assert(8 * (RB / 2) * 4096 <= kLdsBytes && kTileM * (kPfTileN * 2 + 16) <= kLdsBytes, "");
+  // (64-row tiles: 8 KiB of bias sums sit behind the 64 KiB that the swap uses)
+  static_assert(RB != 4 || 65536 + 8192 <= kLdsBytes, "");
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void* p, unsigned bytes) {
@@ -78,6 +80,21 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   constexpr int kPfSlabA = PfShape<RB>::kSlabA;
   constexpr int kPfStageBytes = PfShape<RB>::kStageBytes;
   constexpr int HB = RB / 2;  // row blocks a wave finishes after the halves are added
+  // Per-channel scales with 64-row tiles: every unpacked word meets only four
+  // row blocks, so the loop is bound by the unpack's issue slots (36 VALU to 16
+  // MFMAs per k step), not by the matrix pipe.  There the unpack stops at the
+  // biased integers -- (q & 0x000f000f) | 0x6400 is fp16(1024 + n) and
+  // (q & 0x00f000f0) | 0x5400 is fp16(64 + n) for the nibbles n of a word, five
+  // instructions per word instead of nine -- and the biases and the zero point
+  // (1032 and 72 per activation) are summed by one more MFMA per k step on a
+  // constant weight operand, in a chain of exactly the shape of the weights'
+  // chains, and subtracted at the end: what is left is sum a (n - 8), exact
+  // integers times activations in fp32; a one-hot row returns fp16(n - 8)
+  // exactly, and where every nibble is the zero point the two chains are the
+  // same computation, so the difference is exactly zero.  The four waves of a
+  // k half share the rows, so each sums the bias of one row block (the one it
+  // visits first: wave w walks the row blocks starting from block w).
+  constexpr bool BIAS = !GROUP && RB == 4;
 
   const int kh = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);  // k half
   const int tid = threadIdx.x & 255;  // thread within the half
@@ -146,6 +163,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // LDS slab: [step][k group][row][slot] dwords; chunk x -> step x/4, slot x%4
   const int a_wr = (ax >> 2) * kPfStepBytes + (tid >> 3) * 16 + (ax & 3) * 4;
   const int a_rd = kg * kPlane + nu * 16;
+  // row block visited in turn i: (i + rot) % RB
+  const int rot = BIAS ? wave : 0;
+  auto row_block = [&](int i) { return BIAS ? ((i + rot) & (RB - 1)) : i; };
 
   const DequantConsts dc;
   // this half's stages: [s_begin, s_end) of the K/64 stages; the loop runs the
@@ -197,13 +217,30 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
+  // the biases of the sums of row block `rot` (see BIAS above) and the constant
+  // weight operand that sums them: (1032, 72) per (low, high) nibble pair
+  f4 bias = {0.f, 0.f, 0.f, 0.f};
+  const i4 wbias_i = {0x64086408, 0x54805480, 0x64086408, 0x54805480};
+  const h8 wbias = __builtin_bit_cast(h8, wbias_i);
   h8 w[2][4];  // unpacked weights of the current and the next k step
   i4 af[4];    // ring of activation operands, three ahead of the MFMAs
   i2 bw[2];    // packed weight words of the next k step (its two 16-deep rows)
 
   // unpack the two words of 16-column group j2 of k step (slot, h) into w[buf]
+  const int ex_hi = dc.ex - 0x10001000;  // 0x54005400: fp16(64 + n) for a nibble at bit 4
   auto dequant_pair = [&](int buf, int slot, int h, int j2) {
     (void)h;
+    if constexpr (BIAS) {
+      const int q0 = bw[0][j2], q1 = bw[1][j2];
+      const int r0 = (int)((unsigned)q0 >> 8), r1 = (int)((unsigned)q1 >> 8);
+      const i4 lo = {(q0 & dc.lo_mask) | dc.ex, (q0 & dc.hi_mask) | ex_hi,
+                     (q1 & dc.lo_mask) | dc.ex, (q1 & dc.hi_mask) | ex_hi};
+      const i4 hi = {(r0 & dc.lo_mask) | dc.ex, (r0 & dc.hi_mask) | ex_hi,
+                     (r1 & dc.lo_mask) | dc.ex, (r1 & dc.hi_mask) | ex_hi};
+      w[buf][2 * j2] = __builtin_bit_cast(h8, lo);
+      w[buf][2 * j2 + 1] = __builtin_bit_cast(h8, hi);
+      return;
+    }
     h2 s2 = GROUP ? as_h2(sreg[slot][j2]) : (h2){(half_t)1.f, (half_t)1.f};
     h2 l0, h0, l1, h1, m0_, n0_, m1_, n1_;
     dequant_word<GROUP>(bw[0][j2], s2, dc, l0, h0, l1, h1);
@@ -217,7 +254,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     bw[1] = *(const i2*)(stage_base + b_rd + (2 * h + 1) * 2048);
   };
   auto read_frag = [&](int idx, const char* step_base, int i) {
-    af[idx] = *(const i4*)(step_base + a_rd + i * 256);
+    af[idx] = *(const i4*)(step_base + a_rd + row_block(i) * 256);
   };
 
   // One operation of the unpack of word bw[r][j2] into w[buf] (the sequence of
@@ -235,9 +272,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     switch (op) {
       case 0: wt[r] = (int)((unsigned)q >> 8); break;
       case 1: lo[2 * r] = (q & dc.lo_mask) | dc.ex; break;
-      case 2: lo[2 * r + 1] = (q & dc.hi_mask) | dc.ex; break;
+      case 2: lo[2 * r + 1] = (q & dc.hi_mask) | (BIAS ? ex_hi : dc.ex); break;
       case 3: hi[2 * r] = (wt[r] & dc.lo_mask) | dc.ex; break;
-      case 4: hi[2 * r + 1] = (wt[r] & dc.hi_mask) | dc.ex; break;
+      case 4: hi[2 * r + 1] = (wt[r] & dc.hi_mask) | (BIAS ? ex_hi : dc.ex); break;
       case 5: lo[2 * r] = as_int(as_h2(lo[2 * r]) - sub); break;
       case 6: lo[2 * r + 1] = as_int(__builtin_elementwise_fma(as_h2(lo[2 * r + 1]), mul, add)); break;
       case 7: hi[2 * r] = as_int(as_h2(hi[2 * r]) - sub); break;
@@ -262,7 +299,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // them; scheduling fences keep it that way.  `extra(m)` runs behind MFMA m.
   auto step = [&](int h, const char* cur_base, const char* nxt_base, const char* nxt_stage,
                   int nslot, int nh, auto&& extra) {
-    constexpr int kOpsPerWord = GROUP ? 13 : 9;
+    constexpr int kOpsPerWord = GROUP ? 13 : (BIAS ? 5 : 9);
     constexpr int kPairsPerMfma = RB == 8 ? 1 : 2;  // one operation of each word of a pair
     constexpr int kFirst = RB == 8 ? 6 : 3;         // the words are read from LDS behind MFMA 0
 #pragma unroll
@@ -273,6 +310,9 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
       else
         read_frag((i + 3) & 3, nxt_base, i + 3 - RB);
       const h8 a = __builtin_bit_cast(h8, af[i & 3]);
+      if constexpr (BIAS) {
+        if (i == 0) bias = __builtin_amdgcn_mfma_f32_16x16x32_f16(wbias, a, bias, 0, 0, 0);
+      }
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const int m = 4 * i + j;
@@ -370,6 +410,19 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // slab rings are dead by now.
   const int own = HB * kh;  // first row block this wave finishes
   __syncthreads();
+  if constexpr (BIAS) {
+    // every wave of a k half needs the bias of all four row blocks: wave w has
+    // summed that of block w
+    f4* bx = (f4*)(smem_all + 65536);
+    bx[(kh * 4 + wave) * 64 + lane] = bias;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < RB; i++) {
+      const f4 b = bx[(kh * 4 + row_block(i)) * 64 + lane];
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j] -= b;
+    }
+  }
   {
     f4* out = (f4*)smem_all + (size_t)(kh * 4 + wave) * (HB * 4 * 64);
 #pragma unroll
@@ -460,7 +513,7 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     }
 #pragma unroll
     for (int i = 0; i < HB; i++) {
-      const int m = 16 * (own + i) + nu;
+      const int m = 16 * row_block(own + i) + nu;
       h4 o = {(half_t)fin[i][j][0], (half_t)fin[i][j][1], (half_t)fin[i][j][2],
               (half_t)fin[i][j][3]};
       if (!GROUP) o *= sc;

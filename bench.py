@@ -50,12 +50,18 @@ SHAPES = {
 }
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE and scaled by what the same counters read for a 256 MiB device copy
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this pool); the summaries are under
-# profiles/.  None for workloads not measured.
+# WRITE_SIZE (KiB per dispatch) and scaled by what the same counters read for a
+# 256 MiB device copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this pool); the
+# summaries, with the commands, are under profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "decode": int((4756.5 * 2.0 + 273.0) * 1024),
-    "prefill": int((33371.5 * 2.0 + 16385.3) * 1024),
+    "decode": int((4760.5 * 2.0 + 273.0) * 1024),         # 10.0 MB, 1.16 x algorithmic
+    "batch16": int((5688.5 * 2.0 + 2185.0) * 1024),       # 13.9 MB, 1.56 x (2 MiB of partial sums)
+    "prefill": int((33371.5 * 2.0 + 16393.0) * 1024),     # 85.1 MB, 2.02 x (A and B read by 16 tiles each)
+    "mlp_up": int((12296.0 * 2.0 + 1728.1) * 1024),       # 27.0 MB, 1.14 x
+    "mlp_down": int((13714.5 * 2.0 + 2185.0) * 1024),     # 30.3 MB, 1.28 x
+    "large_g128": int((66886.0 * 2.0 + 17930.5) * 1024),  # 155.3 MB, 1.23 x
+    "large_chan": int((65121.5 * 2.0 + 17930.5) * 1024),  # 151.7 MB, 1.24 x
+    "decode_large": int((59281.0 * 2.0 + 56.0) * 1024),   # 121.5 MB, 1.00 x
 }
 
 

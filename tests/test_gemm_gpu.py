@@ -419,10 +419,11 @@ def test_prefill_kernel_closed_forms(env, rows, slices):
     try:
         assert marlin.plan(M, N, K, 128)[1]["kernel"] == 2
         A = rng.standard_normal((M, K)).astype(np.float16)
-        s = rng.uniform(0.001, 0.02, (K // 128, N)).astype(np.float16)
         q = np.full((K, N), 8, np.uint8)
-        C = gpu_gemm(env, A, O.pack_weights(q), O.pack_scales(s, True), N, C_fill=7.0)
-        assert not C.view(np.uint16).any()
+        for g in (128, -1):
+            s = rng.uniform(0.001, 0.02, (K // 128 if g == 128 else 1, N)).astype(np.float16)
+            C = gpu_gemm(env, A, O.pack_weights(q), O.pack_scales(s, g == 128), N, C_fill=7.0)
+            assert not C.view(np.uint16).any(), g
         Ai = rng.integers(-2, 3, (M, K)).astype(np.float16)
         q = rng.integers(0, 16, (K, N), dtype=np.uint8)
         want = Ai.astype(np.int64) @ (q.astype(np.int64) - 8)
