@@ -13,11 +13,14 @@
 // order and writes C.
 //
 // Kernel: a workgroup of 8 waves (2 x 4, two per SIMD) owns a 256 x 256 tile
-// of C; a wave holds a 128 x 64 fp32 accumulator (128 registers).  With B as
+// of C; a wave holds a 128 x 64 fp32 accumulator (128 registers).  Problems
+// with too few such tiles for the compute units run on 128 x 256 or 128 x 128
+// tiles (same eight waves, a wave's share 64 x 64 or 64 x 32).  With B as
 // the first MFMA operand and A as the second, v_mfma_f32_16x16x32_f16 yields
 // D[n][m]; lane l = 16kg + nu of an operand holds k = 8kg ... 8kg+7 of row nu.
 // Per 64-deep k stage (two MFMA k steps) the workgroup brings a 256 x 64 slab
-// of A and of B into one of two LDS slabs with buffer loads that write LDS
+// of A and of B into a ring of LDS slabs (two; three or four for the smaller
+// tiles, whose stages are shorter than a load's latency) with buffer loads that write LDS
 // directly (16 bytes per lane, lane l at 16*l).  Eight lanes fetch the whole
 // 128-byte k run of a row -- one cache line; with 64-byte runs every line
 // came in twice and the loads alone bounded the kernel -- so a slab is
@@ -25,8 +28,8 @@
 // 16 bytes at chunk 4h + kg of row nu, one ds_read_b128) free of bank
 // conflicts, the chunk stored at position c of row r is chunk c ^ (r % 8);
 // since the hardware fixes where a lane's bytes land, the swizzle is applied
-// to the address the lane fetches.  A slab is requested a whole stage before
-// it is needed; one barrier per stage.  The compiler cannot know which slab a
+// to the address the lane fetches.  A slab is requested at least a whole stage
+// before it is needed; one barrier per stage.  The compiler cannot know which slab a
 // load in flight writes, so the LDS reads of the main loop and their waits are
 // written by hand (LDS reads return in order).
 #include <hip/hip_runtime.h>
@@ -46,18 +49,22 @@ namespace {
 
 constexpr int kDnTile = 256;     // columns of a tile of C, and rows of the large tile
 constexpr int kDnStageK = 64;    // k depth of a stage (two MFMA k steps)
-constexpr int kDnRing = 2;       // slabs in LDS
 constexpr int kDnOob = (int)0x80000000;
 
-// LDS geometry for tiles of TM rows (256, or 128 when the large tiles are too
-// few for the compute units): a slab is TM rows of A and 256 rows of B
-template <int TM>
+// LDS geometry for tiles of TM rows and TN columns (256 x 256; 128 x 256 or
+// 128 x 128 when larger tiles are too few for the compute units): a slab is
+// TM rows of A and TN rows of B
+template <int TM, int TN>
 struct DnShape {
   static constexpr int kSlabA = TM * 128;
-  static constexpr int kSlab = kSlabA + kDnTile * 128;
-  static constexpr int kLds = kDnRing * kSlab;
-  static constexpr int kRB = TM / 32;                 // 16-row blocks per wave
-  static constexpr int kPartBytes = TM * kDnTile * 4;
+  static constexpr int kSlab = kSlabA + TN * 128;
+  // slabs in LDS.  A stage of a small tile is shorter than a load's way from
+  // L2 (0.4 us of MFMAs for 128 x 128), so its slabs are requested further ahead.
+  static constexpr int kRing = TM * TN == 128 * 128 ? 4 : (TM * TN == 128 * 256 ? 3 : 2);
+  static constexpr int kLds = kRing * kSlab;
+  static constexpr int kRB = TM / 32;  // 16-row blocks per wave
+  static constexpr int kNJ = TN / 64;  // 16-column blocks per wave
+  static constexpr int kPartBytes = TM * TN * 4;
 };
 constexpr int kDnMaxSlots = 256;                     // slices in flight per launch
 constexpr int kDnMaxSlices = 4;
@@ -68,6 +75,7 @@ struct DenseArgs {
   void* C;
   int M, N, K;
   int tile_rows;  // 256 or 128
+  int tile_cols;  // 256 or 128
   int tiles_m, tiles_n;
   int dp_tiles;  // tiles computed by one workgroup each
   int sk_tiles;  // tiles (the last ones in tile order) cut into ksplit slices
@@ -123,19 +131,40 @@ __device__ __forceinline__ void dn_wait(i4& v) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(PENDING));
 #endif
 }
+// wait for every LDS read in flight; the operand registers are named so that
+// they count as in use up to here
+__device__ __forceinline__ void drain_reads(i4 (&a)[2], i4 (&b)[2], i4 (&f)[4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(f[0]), "+v"(f[1]), "+v"(f[2]),
+                 "+v"(f[3]));
+#endif
+}
+__device__ __forceinline__ void drain_reads(i4 (&a)[4], i4 (&b)[4], i4 (&f)[4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]),
+                 "+v"(b[3]), "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+#endif
+}
+// s_waitcnt vmcnt(n) lgkmcnt(0) (gfx9 encoding)
+constexpr int dn_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | (0 << 8) | ((n >> 4) << 14); }
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 constexpr int dn_vmcnt(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
 
 }  // namespace
 
-template <int TM>
+template <int TM, int TN>
 __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];  // DnShape<TM>::kLds
-  constexpr int RB = DnShape<TM>::kRB;
-  constexpr int kDnSlabA = DnShape<TM>::kSlabA;
-  constexpr int kDnSlab = DnShape<TM>::kSlab;
-  constexpr int kDnLds = DnShape<TM>::kLds;
-  constexpr int kPart = DnShape<TM>::kPartBytes;
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // DnShape<TM, TN>::kLds
+  using Shape = DnShape<TM, TN>;
+  constexpr int RB = Shape::kRB;
+  constexpr int NJ = Shape::kNJ;
+  constexpr int kDnSlabA = Shape::kSlabA;
+  constexpr int kDnSlab = Shape::kSlab;
+  constexpr int kRing = Shape::kRing;
+  constexpr int kDnLds = Shape::kLds;
+  constexpr int kPart = Shape::kPartBytes;
   __shared__ int s_ticket;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -143,7 +172,7 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   const int kg = lane >> 4;
   const int nu = lane & 15;
   const int wm = wave >> 2;  // row half of the tile
-  const int wn = wave & 3;   // 64-column quarter
+  const int wn = wave & 3;   // column quarter of the tile
 
   // stream-K slices come first in the grid, so that they run beside the first
   // wave of whole tiles
@@ -165,20 +194,21 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   int tm, tn;
   dn_tile_coord(tile, p.tiles_m, p.tiles_n, &tm, &tn);
   const int m0 = tm * TM;
-  const int n0 = tn * kDnTile;
+  const int n0 = tn * TN;
   const int rows = min(TM, p.M - m0);
 
   const __amdgpu_buffer_rsrc_t rA =
       dn_rsrc((const char*)p.A + (size_t)m0 * p.K * 2, (unsigned)rows * (unsigned)p.K * 2u);
   const __amdgpu_buffer_rsrc_t rB =
-      dn_rsrc((const char*)p.B + (size_t)n0 * p.K * 2, (unsigned)kDnTile * (unsigned)p.K * 2u);
+      dn_rsrc((const char*)p.B + (size_t)n0 * p.K * 2, (unsigned)TN * (unsigned)p.K * 2u);
 
-  // wave w fetches rows (TM/8) w ... of the A slab and 32w ... 32w+31 of the
+  // wave w fetches rows (TM/8) w ... of the A slab and (TN/8) w ... of the
   // B slab, eight rows per instruction: lane (r = lane/8, c = lane%8) lands at
   // [r][c] and fetches chunk c ^ r of its row.  Rows past the end of A repeat
   // the last row (never stored).
   constexpr int TA = TM / 64;  // A instructions per wave and stage
-  int a_src[TA], b_src[4];
+  constexpr int TB = TN / 64;  // B instructions per wave and stage
+  int a_src[TA], b_src[TB];
   {
     const int r8 = lane >> 3, c = (lane & 7) ^ r8;
 #pragma unroll
@@ -187,7 +217,7 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
       a_src[t] = (r < rows ? r : rows - 1) * p.K * 2 + 16 * c;
     }
 #pragma unroll
-    for (int t = 0; t < 4; t++) b_src[t] = (32 * wave + 8 * t + r8) * p.K * 2 + 16 * c;
+    for (int t = 0; t < TB; t++) b_src[t] = (8 * TB * wave + 8 * t + r8) * p.K * 2 + 16 * c;
   }
   // this workgroup's stages [st0, st1) of the K/64 stages
   const int stages_all = p.K / kDnStageK;
@@ -204,18 +234,18 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     for (int t = 0; t < TA; t++)
       dn_dma16(rA, base + (8 * TA * wave + 8 * t) * 128, a_src[t] | inv, at);
 #pragma unroll
-    for (int t = 0; t < 4; t++)
-      dn_dma16(rB, base + kDnSlabA + (32 * wave + 8 * t) * 128, b_src[t] | inv, at);
+    for (int t = 0; t < TB; t++)
+      dn_dma16(rB, base + kDnSlabA + (8 * TB * wave + 8 * t) * 128, b_src[t] | inv, at);
   };
-  constexpr int kSlabLoads = TA + 4;  // per wave
+  constexpr int kSlabLoads = TA + TB;  // per wave
 
-  f4 acc[RB][4];
+  f4 acc[RB][NJ];
 #pragma unroll
   for (int i = 0; i < RB; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NJ; j++) acc[i][j] = (f4){0.f, 0.f, 0.f, 0.f};
 
-  i4 w[2][4];  // B operands of the two k steps of a stage
+  i4 w[2][NJ];  // B operands of the two k steps of a stage
   i4 af[4];    // ring of A operands, three ahead of the MFMAs
   // operand addresses in slab 0 for the two k steps
   unsigned a_rd[2], b_rd[2];
@@ -223,18 +253,25 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   for (int h = 0; h < 2; h++) {
     const unsigned sw = 16 * ((4 * h + kg) ^ (nu & 7));
     a_rd[h] = (unsigned)(size_t)smem + (16 * RB * wm + nu) * 128 + sw;
-    b_rd[h] = (unsigned)(size_t)smem + kDnSlabA + (64 * wn + nu) * 128 + sw;
+    b_rd[h] = (unsigned)(size_t)smem + kDnSlabA + (16 * NJ * wn + nu) * 128 + sw;
   }
+  // the NJ B operands of a k step: 16 rows of the slab apart
+  auto read_b = [&](unsigned at, i4 (&dst)[NJ]) {
+    dn_read16<0>(at, dst[0]);
+    dn_read16<2048>(at, dst[1]);
+    if constexpr (NJ == 4) {
+      dn_read16<4096>(at, dst[2]);
+      dn_read16<6144>(at, dst[3]);
+    }
+  };
 
-  // prologue: slabs 0 and 1 requested; slab 0 landed; its first operands read
-  issue_slab(0, 0);
-  issue_slab(1, 1);
-  __builtin_amdgcn_s_waitcnt(dn_vmcnt(kSlabLoads));
+  // prologue: slabs 0 ... kRing-1 requested; slab 0 landed (loads complete in
+  // order); its first operands read
+#pragma unroll
+  for (int r = 0; r < kRing; r++) issue_slab(r, r);
+  __builtin_amdgcn_s_waitcnt(dn_vmcnt((kRing - 1) * kSlabLoads));
   __builtin_amdgcn_s_barrier();
-  dn_read16<0>(b_rd[0], w[0][0]);
-  dn_read16<2048>(b_rd[0], w[0][1]);
-  dn_read16<4096>(b_rd[0], w[0][2]);
-  dn_read16<6144>(b_rd[0], w[0][3]);
+  read_b(b_rd[0], w[0]);
   dn_read16<0>(a_rd[0], af[0]);
   dn_read16<2048>(a_rd[0], af[1]);
   dn_read16<4096>(a_rd[0], af[2]);
@@ -242,16 +279,16 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   // One k step (H) of the stage in slab `cur`.  LDS reads in issue order, with
   // Ai the operand of row block i and primes the prefetches for the step after
   // (eight row blocks per wave; with four the same three-ahead pattern):
-  //   step 0:  | B(step 1) x4  A3 | A4 | A5 | A6 | A7 | A0' | A1' | A2' |
-  //   step 1:  | A3 | A4 | A5 | A6 | A7 | barrier, B(next stage) x4  A0' | A1' | A2' |
+  //   step 0:  | B(step 1) x NJ  A3 | A4 | A5 | A6 | A7 | A0' | A1' | A2' |
+  //   step 1:  | A3 | A4 | A5 | A6 | A7 | barrier, B(next stage) x NJ  A0' | A1' | A2' |
   // When row block i is used, the reads issued after Ai may still be pending:
-  // three A operands, plus the four B reads where those were issued in between
+  // three A operands, plus the NJ B reads where those were issued in between
   // (the three row blocks from the one that issues them).
   // The barrier of a stage sits where the first read from the next slab is
   // about to be issued: by then every wave has its own part of that slab (it
   // waits for its loads first) and has issued and received all its reads of
   // the current slab, which the request for the stage after next overwrites.
-  auto kstep = [&](auto H, unsigned cur, unsigned nxt, int s) {
+  auto kstep = [&](auto H, unsigned cur, unsigned nxt, int s, int slot) {
     constexpr int h = decltype(H)::value;
     constexpr int ib = h ? RB - 3 : 0;  // row block that issues the B reads
     const unsigned ac = a_rd[h] + cur;                        // this step, this slab
@@ -261,14 +298,13 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     for (int i = 0; i < RB; i++) {
       if (i == ib) {
         if (h == 1) {
-          __builtin_amdgcn_s_waitcnt(0);  // my loads of the next slab and my reads of this one
+          // my loads of the next slab (the slabs after it may still be on
+          // their way) and my reads of this one
+          __builtin_amdgcn_s_waitcnt(dn_vm_lgkm0((kRing - 2) * kSlabLoads));
           __builtin_amdgcn_s_barrier();
-          issue_slab(s + 2, (int)(cur != 0));
+          issue_slab(s + kRing, slot);
         }
-        dn_read16<0>(bn, w[h ^ 1][0]);
-        dn_read16<2048>(bn, w[h ^ 1][1]);
-        dn_read16<4096>(bn, w[h ^ 1][2]);
-        dn_read16<6144>(bn, w[h ^ 1][3]);
+        read_b(bn, w[h ^ 1]);
       }
       // operand of row block i + 3: of this step, or of the step after
       auto frag = [&](auto I) {
@@ -289,27 +325,37 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
         case 7: frag(std::integral_constant<int, 10>{}); break;
       }
       if (i >= ib && i <= ib + 2)
-        dn_wait<7>(af[i & 3]);
+        dn_wait<3 + NJ>(af[i & 3]);
       else
         dn_wait<3>(af[i & 3]);
       if (i == 0) {
         // the B operands of this step were requested before A0 was
 #pragma unroll
-        for (int j = 0; j < 4; j++) asm volatile("" : "+v"(w[h][j]));
+        for (int j = 0; j < NJ; j++) asm volatile("" : "+v"(w[h][j]));
       }
       const h8 a = __builtin_bit_cast(h8, af[i & 3]);
 #pragma unroll
-      for (int j = 0; j < 4; j++)
+      for (int j = 0; j < NJ; j++)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, w[h][j]), a,
                                                            acc[i][j], 0, 0, 0);
     }
   };
 
+  int slot = 0;  // ring slot of the stage being computed
   for (int s = 0; s < stages; s++) {
-    const unsigned cur = (s & 1) ? kDnSlab : 0, nxt = (s & 1) ? 0 : kDnSlab;
-    kstep(std::integral_constant<int, 0>{}, cur, nxt, s);
-    kstep(std::integral_constant<int, 1>{}, cur, nxt, s);
+    const int slot_next = slot == kRing - 1 ? 0 : slot + 1;
+    const unsigned cur = slot * kDnSlab, nxt = slot_next * kDnSlab;
+    kstep(std::integral_constant<int, 0>{}, cur, nxt, s, slot);
+    kstep(std::integral_constant<int, 1>{}, cur, nxt, s, slot);
+    slot = slot_next;
   }
+  // The last k step has requested the operands of a stage that does not
+  // exist; they are still on their way into w and af.  Those registers stay
+  // taken until the reads have landed: the compiler, which believes they were
+  // written when the reads were issued and sees no further use, would
+  // otherwise hand them to the code below at once, and a late arrival would
+  // overwrite what that code keeps there.
+  drain_reads(w[0], w[1], af);
   // Nothing of the ring may still be on its way when LDS is reused.
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
@@ -320,14 +366,14 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
   // slices in slice order (its own from registers at its place in that order).
   if (ksplit > 1) {
     const __amdgpu_buffer_rsrc_t rP = dn_rsrc(p.scratch, 0x7fffffffu);
-    const int at = (wave * (RB * 4) * 64 + lane) * 16;
+    const int at = (wave * (RB * NJ) * 64 + lane) * 16;
     const int mine = work * kPart;
 #pragma unroll
     for (int i = 0; i < RB; i++)
 #pragma unroll
-      for (int j = 0; j < 4; j++)
+      for (int j = 0; j < NJ; j++)
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4, acc[i][j]), rP,
-                                               at + (i * 4 + j) * 1024, mine, 16 /* sc1 */);
+                                               at + (i * NJ + j) * 1024, mine, 16 /* sc1 */);
     __builtin_amdgcn_s_waitcnt(dn_vmcnt(0));  // my stores have been acknowledged
     __syncthreads();
     const int sk_tile = tile - p.dp_tiles;
@@ -340,19 +386,19 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
     // together, then added in slice order with my own at its place
 #pragma unroll
     for (int i = 0; i < RB; i++) {
-      f4 v[kDnMaxSlices][4];
+      f4 v[kDnMaxSlices][NJ];
 #pragma unroll
       for (int k2 = 0; k2 < kDnMaxSlices; k2++) {
         const int theirs = (sk_tile * ksplit + k2) * kPart;
         const int inv = (k2 < ksplit && k2 != ks) ? 0 : kDnOob;  // no traffic for the rest
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NJ; j++)
           v[k2][j] = __builtin_bit_cast(
-              f4, __builtin_amdgcn_raw_buffer_load_b128(rP, (at + (i * 4 + j) * 1024) | inv,
+              f4, __builtin_amdgcn_raw_buffer_load_b128(rP, (at + (i * NJ + j) * 1024) | inv,
                                                         theirs, 16 /* sc1 */));
       }
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
+      for (int j = 0; j < NJ; j++) {
         f4 sum = (ks == 0) ? acc[i][j] : v[0][j];
 #pragma unroll
         for (int k2 = 1; k2 < kDnMaxSlices; k2++)
@@ -366,10 +412,12 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
 
   // ---- C: a lane holds, per (i, j), row 16i + nu and four consecutive
   // columns.  The fp16 tile goes through LDS (the slabs are dead), one half of
-  // its rows at a time, and leaves as whole 512-byte rows with 16-byte stores;
-  // 8-byte stores straight from the registers cost 13 us more at 4096^3.
-  constexpr int kPitch = kDnTile * 2 + 16;  // bytes per tile row in LDS
-  constexpr int HR = TM / 2;                // rows of a half
+  // its rows at a time, and leaves as whole rows (512 or 256 bytes) with
+  // 16-byte stores; 8-byte stores straight from the registers cost 13 us more
+  // at 4096^3.
+  constexpr int kPitch = TN * 2 + 16;  // bytes per tile row in LDS
+  constexpr int HR = TM / 2;           // rows of a half
+  constexpr int PR = TN / 8;           // 16-byte pieces of a row
   static_assert(HR * kPitch <= kDnLds, "");
   half_t* C = (half_t*)p.C;
   const int q = lane >> 4;
@@ -380,17 +428,17 @@ __global__ __launch_bounds__(512) void dense_kernel(DenseArgs p) {
 #pragma unroll
       for (int i = 0; i < RB; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NJ; j++) {
           const h4 o = {(half_t)acc[i][j][0], (half_t)acc[i][j][1], (half_t)acc[i][j][2],
                         (half_t)acc[i][j][3]};
-          *(h4*)(smem + (16 * i + nu) * kPitch + (64 * wn + 16 * j + 4 * q) * 2) = o;
+          *(h4*)(smem + (16 * i + nu) * kPitch + (16 * NJ * wn + 16 * j + 4 * q) * 2) = o;
         }
     }
     __syncthreads();
 #pragma unroll
-    for (int it = 0; it < HR / 16; it++) {
+    for (int it = 0; it < HR * PR / 512; it++) {
       const int piece = it * 512 + tid;  // 16-byte piece of the half tile
-      const int r = piece >> 5, c16 = piece & 31;
+      const int r = piece / PR, c16 = piece % PR;
       const int m = HR * hlf + r;
       if (m < rows) {
         const i4 v = *(const i4*)(smem + r * kPitch + c16 * 16);
@@ -436,7 +484,7 @@ std::mutex g_dn_mu;
 DnDevice g_dn[kDnMaxDevices];
 
 struct DnPlan {
-  int tile_rows, tiles_m, tiles_n, dp_tiles, sk_tiles, ksplit, grid;
+  int tile_rows, tile_cols, tiles_m, tiles_n, dp_tiles, sk_tiles, ksplit, grid;
 };
 
 // Whole waves of tiles go to one workgroup each; the tiles of the partial last
@@ -446,10 +494,16 @@ struct DnPlan {
 DnPlan dn_plan(int m, int n, int k, int cus) {
   DnPlan pl;
   // 256 x 256 tiles, unless they would occupy at most half of the compute
-  // units: then 128 x 256 tiles, twice as many
-  pl.tile_rows = (2LL * ceil_div(m, kDnTile) * (n / kDnTile) <= cus) ? 128 : kDnTile;
+  // units: then 128 x 256 tiles, twice as many, and 128 x 128 if that holds
+  // for those as well (one workgroup per smaller tile beats k slices of a
+  // larger one: no partial sums go through memory)
+  pl.tile_rows = pl.tile_cols = kDnTile;
+  if (2LL * ceil_div(m, kDnTile) * (n / kDnTile) <= cus) {
+    pl.tile_rows = 128;
+    if (2LL * ceil_div(m, 128) * (n / kDnTile) <= cus) pl.tile_cols = 128;
+  }
   pl.tiles_m = ceil_div(m, pl.tile_rows);
-  pl.tiles_n = n / kDnTile;
+  pl.tiles_n = n / pl.tile_cols;
   const int tiles = pl.tiles_m * pl.tiles_n;
   const int rem = cus > 0 ? tiles % cus : 0;
   int s = 1;
@@ -528,11 +582,17 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
       }
       cus = d.cus;
       if (!d.configured) {
-        e = hipFuncSetAttribute((const void*)dense_kernel<256>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, DnShape<256>::kLds);
+        e = hipFuncSetAttribute((const void*)dense_kernel<256, 256>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                DnShape<256, 256>::kLds);
         if (e == hipSuccess)
-          e = hipFuncSetAttribute((const void*)dense_kernel<128>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, DnShape<128>::kLds);
+          e = hipFuncSetAttribute((const void*)dense_kernel<128, 256>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  DnShape<128, 256>::kLds);
+        if (e == hipSuccess)
+          e = hipFuncSetAttribute((const void*)dense_kernel<128, 128>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  DnShape<128, 128>::kLds);
         if (e != hipSuccess) {
           dn_set_error(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
           break;
@@ -545,7 +605,7 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     ScratchView view = {nullptr, nullptr};
     if (pl.sk_tiles > 0 &&
         !scratch_acquire(dev, stream,
-                         (size_t)pl.sk_tiles * pl.ksplit * pl.tile_rows * kDnTile * 4, &view,
+                         (size_t)pl.sk_tiles * pl.ksplit * pl.tile_rows * pl.tile_cols * 4, &view,
                          g_dn_error, sizeof(g_dn_error)))
       break;
     (void)hipGetLastError();  // an earlier call's error is not this launch's
@@ -557,6 +617,7 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.N = n;
     a.K = k;
     a.tile_rows = pl.tile_rows;
+    a.tile_cols = pl.tile_cols;
     a.tiles_m = pl.tiles_m;
     a.tiles_n = pl.tiles_n;
     a.dp_tiles = pl.dp_tiles;
@@ -564,10 +625,14 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
     a.ksplit = pl.ksplit;
     a.locks = view.counters;
     a.scratch = view.partials;
-    if (pl.tile_rows == 128)
-      hipLaunchKernelGGL(dense_kernel<128>, dim3(pl.grid), dim3(512), DnShape<128>::kLds, stream, a);
+    constexpr int lds_small = DnShape<128, 128>::kLds, lds_half = DnShape<128, 256>::kLds,
+                  lds_large = DnShape<256, 256>::kLds;
+    if (pl.tile_cols == 128)
+      hipLaunchKernelGGL((dense_kernel<128, 128>), dim3(pl.grid), dim3(512), lds_small, stream, a);
+    else if (pl.tile_rows == 128)
+      hipLaunchKernelGGL((dense_kernel<128, 256>), dim3(pl.grid), dim3(512), lds_half, stream, a);
     else
-      hipLaunchKernelGGL(dense_kernel<256>, dim3(pl.grid), dim3(512), DnShape<256>::kLds, stream, a);
+      hipLaunchKernelGGL((dense_kernel<256, 256>), dim3(pl.grid), dim3(512), lds_large, stream, a);
     e = hipGetLastError();
     if (e != hipSuccess) {
       dn_set_error(e, "kernel launch");
@@ -592,6 +657,7 @@ int streamk_amd_plan(int m, int n, int k, int cus, int* out) {
   out[4] = pl.ksplit;
   out[5] = pl.grid;
   out[6] = pl.tile_rows;
+  out[7] = pl.tile_cols;
   return STREAMK_OK;
 }
 

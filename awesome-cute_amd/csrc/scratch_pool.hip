@@ -90,9 +90,12 @@ bool scratch_acquire(int dev, hipStream_t stream, size_t partial_bytes, ScratchV
       fail(err, err_len, "hipMalloc(scratch)", e);
       return false;
     }
-    e = hipMemset(p, 0, kCounterBytes);
+    // Cleared on the caller's stream, ahead of the launch that will use the
+    // counters: a clear on the null stream is not ordered against a
+    // non-blocking stream and could land in the middle of that launch.
+    e = hipMemsetAsync(p, 0, kCounterBytes, stream);
     if (e != hipSuccess) {
-      fail(err, err_len, "hipMemset(scratch)", e);
+      fail(err, err_len, "hipMemsetAsync(scratch)", e);
       (void)hipFree(p);
       return false;
     }

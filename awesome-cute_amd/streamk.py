@@ -32,10 +32,10 @@ def check(m, n, k):
 
 
 def plan(m, n, k, cus=256):
-    """The split of the output tiles (tile_rows x 256) into data-parallel and stream-K tiles."""
-    out = (ctypes.c_int * 7)()
+    """The split of the output tiles (tile_rows x tile_cols) into data-parallel and stream-K tiles."""
+    out = (ctypes.c_int * 8)()
     rc = _lib.streamk_amd_plan(m, n, k, cus, out)
-    keys = ("tiles_m", "tiles_n", "dp_tiles", "sk_tiles", "k_slices", "grid", "tile_rows")
+    keys = ("tiles_m", "tiles_n", "dp_tiles", "sk_tiles", "k_slices", "grid", "tile_rows", "tile_cols")
     return rc, dict(zip(keys, out))
 
 

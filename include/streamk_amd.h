@@ -26,7 +26,7 @@ extern "C" {
  * fp32 accumulation.  m is arbitrary; n % 256 == 0 and k % 64 == 0.
  * Partial sums of the stream-K tiles live in the library-owned buffer of this
  * (device, stream) that marlin_gemm uses too (include/marlin_amd.h): sized by
- * the launch (256 KiB per slice of a stream-K tile), grown on demand, none for
+ * the launch (tile rows x tile columns x 4 bytes per slice of a stream-K tile), grown on demand, none for
  * launches without stream-K tiles.  Calls on one stream may follow each other
  * freely, calls that overlap must use different streams; a call that would have
  * to allocate under graph capture returns STREAMK_ERR_RUNTIME. */
@@ -37,11 +37,12 @@ int streamk_gemm_tn(const void* A, const void* B, void* C, int m, int n, int k, 
 int streamk_amd_check(int m, int n, int k);
 
 /* the tile split for a device with `cus` compute units (counterpart of
- * SK_DP_Block_Wrapper, dp_sk_block.h:31-80): out[0..6] = tiles along m, tiles
+ * SK_DP_Block_Wrapper, dp_sk_block.h:31-80): out[0..7] = tiles along m, tiles
  * along n (tiles numbered in panels of 8 column tiles), data-parallel tiles, stream-K
  * tiles (the last ones in tile order), k slices per stream-K tile, workgroups,
  * rows of a tile (256, or 128 when 256 x 256 tiles would occupy at most half
- * of the compute units; tiles are 256 columns wide) */
+ * of the compute units), columns of a tile (256, or 128 when 128 x 256 tiles
+ * would occupy at most half of them too) */
 int streamk_amd_plan(int m, int n, int k, int cus, int* out);
 
 /* out[0], out[1] = row and column tile of tile number `tile` (0 <= tile <

@@ -235,6 +235,42 @@ def test_two_streams_run_side_by_side(env):
             assert not ws.any().item()
 
 
+def test_kernels_of_other_streams_beside_do_not_change_the_result(env):
+    """A launch gives the same bits whatever else runs on the GPU: kernels of another
+    stream that keep LDS and memory busy stretch every latency inside the GEMM, which
+    must not matter (shared column tiles of the streaming kernel with 1, 16 and 64 rows,
+    k slices of the prefill kernel)."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    shapes = [(1, 4096, 4096, 51), (16, 2048, 8192, 52), (64, 4096, 4096, 53), (128, 4096, 4096, 54)]
+    x = torch.randn(4096, 4096, device=dev)
+    beside, main = torch.cuda.Stream(), torch.cuda.Stream()
+    for (m, n, k, seed) in shapes:
+        A, q, s, B, sp = O.make_problem(m, n, k, 128, seed)
+        dA, dB, ds = (torch.from_numpy(v).to(dev) for v in (A, B, sp))
+
+        def run():
+            dC = torch.zeros((m, n), dtype=torch.half, device=dev)
+            ws = torch.zeros(n // 128 * 16, dtype=torch.int, device=dev)
+            marlin.mul(dA, dB, dC, ds, ws)
+            return dC
+
+        alone = run()
+        torch.cuda.synchronize()
+        outs = []
+        for it in range(20):
+            with torch.cuda.stream(beside):
+                if it % 2:
+                    torch.sort(x[:512], dim=1)
+                else:
+                    for _ in range(3):
+                        torch.softmax(x, dim=1)
+            with torch.cuda.stream(main):
+                outs.append(run())
+        torch.cuda.synchronize()
+        assert all(torch.equal(c, alone) for c in outs), (m, n, k)
+
+
 def test_two_host_threads_two_streams(env):
     """Two host threads, each with a stream of its own, call the library at the same time
     (ctypes releases the interpreter lock during a call): the per-device state behind the

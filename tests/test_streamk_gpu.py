@@ -59,10 +59,12 @@ def close(C, ref):
     assert cos >= 0.999
 
 
-# one tile; row tails; several tiles; stream-K tiles with 2, 3 and 4 slices on 256 CUs
+# one tile; row tails; several tiles; stream-K tiles with 2, 3 and 4 slices on 256 CUs;
+# 128 x 128 tiles (few tiles), 128 x 256 (640 x 7424) and 256 x 256 (1100 x 8192)
 SHAPES = [(256, 256, 64), (1, 256, 64), (16, 256, 192), (255, 256, 128), (257, 512, 320),
           (300, 512, 1024), (256, 512, 4096), (700, 768, 1024), (512, 256, 2048),
-          (1000, 2816, 512), (640, 7424, 512)]
+          (1000, 2816, 512), (640, 7424, 512), (129, 256, 512), (200, 512, 768),
+          (1024, 1024, 1024), (1100, 8192, 128)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -97,7 +99,8 @@ def test_one_hot_rows_return_rows_of_b(env):
 
 
 @pytest.mark.parametrize("m,n,k", [(4096, 4352, 4096), (1152, 4352, 4096), (4096, 4352, 10240),
-                                   (4000, 4352, 512), (8100, 8192, 256)])
+                                   (4000, 4352, 512), (8100, 8192, 256), (2048, 2048, 2048),
+                                   (1000, 4096, 4096)])
 def test_reference_examples(env, m, n, k):
     """The reference's stream-K examples at full size (gemm/readme.md:27-31), and two
     shapes whose last row tile of 256 is partly empty: a sample of rows against the oracle, the whole result against torch's fp32 product by the
@@ -157,6 +160,35 @@ def test_two_streams_run_side_by_side(env):
     torch.cuda.synchronize()
     for c1, c2 in outs:
         assert torch.equal(c1, alone[0]) and torch.equal(c2, alone[1])
+
+
+@pytest.mark.parametrize("m,n,k", [(700, 768, 1024), (512, 256, 2048), (2048, 2048, 512)])
+def test_kernels_of_other_streams_beside_do_not_change_the_result(env, m, n, k):
+    """A launch must give the same bits whatever else runs on the GPU.  Kernels of another
+    stream that keep the compute units' LDS and memory busy (softmax, sort) stretch the
+    latencies inside the GEMM; once, operand reads still in flight when the main loop ended
+    landed in registers that already held the addresses of the partial sums."""
+    torch, streamk = env
+    dev = torch.device("cuda:0")
+    A, B = inputs(m, n, k, 5)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev)
+    alone = streamk.gemm(dA, dB)
+    torch.cuda.synchronize()
+    x = torch.randn(4096, 4096, device=dev)
+    beside, main = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    for it in range(30):
+        with torch.cuda.stream(beside):
+            if it % 2:
+                torch.sort(x[:512], dim=1)
+            else:
+                for _ in range(3):
+                    torch.softmax(x, dim=1)
+        with torch.cuda.stream(main):
+            outs.append(streamk.gemm(dA, dB))
+    torch.cuda.synchronize()
+    assert all(torch.equal(c, alone) for c in outs)
+    close(alone.cpu().numpy(), O.dense_gemm_tn(A, B))
 
 
 def test_degenerate_sizes_and_errors(env):

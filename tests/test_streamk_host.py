@@ -54,10 +54,13 @@ def test_tile_split_properties(streamk, cus):
     for m, n, k in cases:
         rc, p = streamk.plan(m, n, k, cus)
         assert rc == 0
-        # 256 x 256 tiles, or 128 x 256 when the large ones would fill at most half the CUs
+        # 256 x 256 tiles; 128 x 256 when those would fill at most half the CUs; 128 x 128
+        # when the 128 x 256 ones would, too
         large = -(-m // 256) * (n // 256)
+        half = -(-m // 128) * (n // 256)
         assert p["tile_rows"] == (128 if 2 * large <= cus else 256)
-        tiles = -(-m // p["tile_rows"]) * (n // 256)
+        assert p["tile_cols"] == (128 if 2 * large <= cus and 2 * half <= cus else 256)
+        tiles = -(-m // p["tile_rows"]) * (n // p["tile_cols"])
         assert p["tiles_m"] * p["tiles_n"] == tiles
         assert p["dp_tiles"] + p["sk_tiles"] == tiles
         assert p["grid"] == p["dp_tiles"] + p["sk_tiles"] * p["k_slices"]
@@ -85,7 +88,12 @@ def test_reference_shapes_use_the_stream_k_tail(streamk):
         assert rc == 0 and p["tile_rows"] == 256
         assert p["dp_tiles"] == 256 and p["sk_tiles"] == 16 and p["k_slices"] == 4, (m, n, k, p)
     rc, p = streamk.plan(1152, 4352, 4096, 256)
-    assert rc == 0 and p["tile_rows"] == 128 and p["dp_tiles"] + p["sk_tiles"] == 9 * 17
+    assert rc == 0 and (p["tile_rows"], p["tile_cols"]) == (128, 256)
+    assert p["dp_tiles"] + p["sk_tiles"] == 9 * 17
+    # so few tiles that 128 x 128 ones fill the compute units without any k slices
+    rc, p = streamk.plan(2048, 2048, 2048, 256)
+    assert rc == 0 and (p["tile_rows"], p["tile_cols"]) == (128, 128)
+    assert p["dp_tiles"] == 256 and p["sk_tiles"] == 0
     rc, p = streamk.plan(4096, 4096, 4096, 256)
     assert p["sk_tiles"] == 0 and p["dp_tiles"] == 256 and p["tile_rows"] == 256
 
