@@ -47,7 +47,16 @@ SHAPES = {
     # not one of the benchmark's configurations: the decode kernel where the
     # launch and exchange latencies are small beside the weight stream
     "decode_large": (1, 28672, 8192, 128, "hbm"),
+    # the row counts between the benchmark's configurations, N = K = 4096 (reported
+    # under "m_sweep": which kernel the host picks and what it costs)
+    "m32": (32, 4096, 4096, 128, "hbm"),
+    "m64": (64, 4096, 4096, 128, "hbm"),
+    "m128": (128, 4096, 4096, 128, "hbm"),
+    "m256": (256, 4096, 4096, 128, "mfma"),
+    "m512": (512, 4096, 4096, 128, "mfma"),
+    "m1024": (1024, 4096, 4096, 128, "mfma"),
 }
+M_SWEEP = ["m32", "m64", "m128", "m256", "m512", "m1024"]
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (KiB per dispatch) and scaled by what the same counters read for a
@@ -323,14 +332,28 @@ def main():
         if main_name == "decode" else None,
     }
     if args.shape == "headline":
+        sweep = []
+        for n in M_SWEEP:
+            r = time_shape(torch, marlin, O, n, min(args.steps, 400), args.warmup)
+            rc, plan = marlin.plan(r["M"], r["N"], r["K"], r["groupsize"], -1, -1, -1,
+                                   info["compute_units"])
+            sweep.append({"M": r["M"], "N": r["N"], "K": r["K"], "groupsize": r["groupsize"],
+                          "us_per_launch": r["us_per_launch"], "weight_GBps": r["weight_GBps"],
+                          "tflops": r["tflops"],
+                          "kernel": {1: "stream", 2: "prefill"}.get(plan["kernel"]),
+                          "grid": plan["grid"], "k_slices": plan["k_slices"],
+                          "tile_rows": plan["tile_rows"]})
+        out["m_sweep"] = sweep
         # the sibling dense fp16 GEMM with its stream-K tail, on the reference's three
-        # examples (gemm/readme.md:29-31); its own program is gemm_streamk.py
+        # examples (gemm/readme.md:29-31) and one problem small enough for 128 x 128
+        # tiles; its own program is gemm_streamk.py
         import gemm_streamk
         out["dense_streamk"] = [
             {k: v for k, v in gemm_streamk.run(m, n, k, repeat=50, log=lambda *_: None).items()
              if k in ("value", "unit", "ms_per_step", "config", "roofline", "vendor_library_tflops",
                       "cos_similarity", "check")}
-            for (m, n, k) in [(4096, 4352, 4096), (4096, 4352, 10240), (1152, 4352, 4096)]]
+            for (m, n, k) in [(4096, 4352, 4096), (4096, 4352, 10240), (1152, 4352, 4096),
+                              (2048, 2048, 2048)]]
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(O, main_name)
     print(json.dumps(out))
