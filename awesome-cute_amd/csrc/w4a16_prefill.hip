@@ -13,18 +13,19 @@
 // Within a half, wave w keeps a 16*RB x 64 fp32 accumulator (16*RB registers):
 // columns 16j+8h+c of the two 64-column blocks 2p, 2p+1 with p = w/2 and
 // j in {2(w%2), 2(w%2)+1}.
-//   - Weights never touch LDS: each lane reads the 8 bytes of its Marlin
-//     16-byte piece that belong to its two 16-column groups straight from
-//     global memory (L2-resident after the first row tile), unpacks them in
-//     registers and feeds them to the MFMA as the first operand.  One unpack
-//     serves eight MFMAs (the eight 16-row blocks).
+//   - Packed weights are copied to LDS as they lie in memory (coalesced
+//     16-byte loads, four 2 KiB rows per stage and half); each lane then picks
+//     the 8 bytes of its Marlin 16-byte piece that belong to its two 16-column
+//     groups, unpacks them in registers and feeds them to the MFMA as the
+//     first operand.  One unpack serves the RB MFMAs of the tile's row blocks.
 //   - Activations are shared by the four waves of a half: they stage a
-//     128 x 64 fp16 slab per k stage through a ring of three LDS buffers,
+//     16*RB x 64 fp16 slab per k stage through a ring of three LDS buffers,
 //     stored in the k-slot order the weight layout dictates so that an
 //     operand is one conflict-free ds_read_b128.
-// Per 32-deep k step a wave issues 32 MFMAs, 8 LDS reads and the unpack of 4
-// weight words (52 VALU instructions), software-pipelined one step ahead and
-// dealt out two behind every MFMA, where they cost no issue time.
+// Per 32-deep k step a wave issues 4*RB MFMAs, RB + 2 LDS reads and the unpack
+// of 4 weight words (52 VALU instructions with group scales), software-
+// pipelined one step ahead and dealt out behind the MFMAs, two (RB = 8) or
+// four (RB = 4) per MFMA.
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
