@@ -142,14 +142,18 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
   // Packed weights go through LDS too: the 256 threads of a half copy the
   // stage's four 2 KiB rows with coalesced 16-byte loads, and every lane then
   // picks its 8 bytes (Marlin piece (t = kg, c = nu%8) of block 2p + nu/8,
-  // words 2jp, 2jp+1).  Pieces are rotated inside each group of four so that
-  // those reads are free of bank conflicts.
+  // words 2jp, 2jp+1).  In LDS the two halves of the pieces of a pair of
+  // 64-column blocks lie apart -- 64 x 8 bytes of words 0,1, then 64 x 8 bytes
+  // of words 2,3 -- so that the 64 lanes of a wave read 512 contiguous bytes,
+  // and the pieces are rotated inside each group of four so that each half of
+  // the wave touches every bank once (with the halves interleaved a wave used
+  // half of the banks: 12 cycles per read instead of 4).
   const int bx = tid & 127;  // 16-byte piece inside a row, for the copy
   const int b_ld = 2048 * tn + 16 * bx;
   const int b_a = (bx & 63) >> 2;
   const int b_wr = kPfSlabA + (wave >> 1) * 2048 + (bx >> 6) * 1024 +
-                   16 * (4 * b_a + (((bx & 3) + (b_a >> 2)) & 3));
-  const int b_rd = kPfSlabA + pr * 1024 + 16 * (4 * nu + ((kg + (nu >> 2)) & 3)) + 8 * jp;
+                   8 * (4 * b_a + (((bx & 3) + (b_a >> 2)) & 3));
+  const int b_rd = kPfSlabA + pr * 1024 + 8 * (4 * nu + ((kg + (nu >> 2)) & 3)) + 512 * jp;
   const int s_lane = (256 * tn + 128 * pr + 8 * nu) * 2 + 8 * jp;
 
   // slab staging: thread (row = tid/8 + 32 i, chunk x = tid%8) moves 16 bytes;
@@ -209,7 +213,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
       for (int g = 0; g < 4; g++) *(int*)(base + a_wr + g * kPlane + i * 32 * 16) = areg[i][g];
 #pragma unroll
-    for (int i = 0; i < 2; i++) *(i4*)(base + b_wr + i * 4096) = bcopy[i];
+    for (int i = 0; i < 2; i++) {
+      *(i2*)(base + b_wr + i * 4096) = (i2){bcopy[i][0], bcopy[i][1]};
+      *(i2*)(base + b_wr + i * 4096 + 512) = (i2){bcopy[i][2], bcopy[i][3]};
+    }
   };
 
   f4 acc[RB][4];
@@ -354,7 +361,10 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
     } else {
       const int y = x - HB * kPerA, i = y >> 1;
       if ((y & 1) == 0)
-        *(i4*)(base + b_wr + i * 4096) = bcopy[i];
+      {
+        *(i2*)(base + b_wr + i * 4096) = (i2){bcopy[i][0], bcopy[i][1]};
+        *(i2*)(base + b_wr + i * 4096 + 512) = (i2){bcopy[i][2], bcopy[i][3]};
+      }
       else
         bcopy[i] = __builtin_amdgcn_raw_buffer_load_b128(
             rB, b_ld | inv, (4 * sg + 2 * i + (wave >> 1)) * b_row, 0);
