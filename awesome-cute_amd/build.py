@@ -1,6 +1,7 @@
 """Builds libmarlin_amd.so (HIP kernels + C ABI) in-tree for gfx950."""
 import os
 import subprocess
+import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -14,11 +15,12 @@ SOURCES = {
     "w4a16_stream.hip": [],
     "w4a16_probe.hip": [],
     "w4a16_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "w4a16_prefill_wide.hip": [],
     "f16_streamk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I", os.path.join(HERE, "build"),
     # packed fp32 arithmetic stays off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
@@ -39,6 +41,10 @@ def _run(cmd, verbose):
 def build_library(verbose=False):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
+    # the assembly statements of the four-wave prefill kernel (prologue, main
+    # loop and accumulator hand-over with fixed registers) are written by a
+    # generator; w4a16_prefill_wide.hip includes them from the build directory
+    _run([sys.executable, os.path.join(CSRC, "gen_prefill_wide.py"), objdir], verbose)
     objs = []
     for src, extra in SOURCES.items():
         obj = os.path.join(objdir, src.replace(".hip", ".o"))

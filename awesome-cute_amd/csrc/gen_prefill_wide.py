@@ -1,0 +1,367 @@
+#!/usr/bin/env python3
+"""Writes the main loop of the four-wave prefill kernel (w4a16_prefill_wide.hip)
+as one inline-assembly statement with fixed registers.
+
+Why assembly: a wave of that kernel owns a 128 x 128 fp32 accumulator, i.e. all
+256 AGPRs, next to about 170 live VGPRs.  With no register to spare the
+compiler's allocator moves accumulators around and spills inside the loop; with
+the registers named here nothing moves.  The schedule is also exactly the one
+written down here: which unpack operation, LDS access or load is issued behind
+which MFMA, and every s_waitcnt is computed from the order of issue.
+
+The statement covers prologue, loop and the first part of the epilogue:
+  prologue  requests of stages 0 and 1, slab 0 to LDS, unpack of the first k step
+  loop      two 64-deep stages per turn (stage parity u is static), see stage()
+  epilogue  row blocks 4..7 of the accumulator go to LDS for the other k half,
+            row blocks 0..3 to v[0:127], which are the statement's outputs
+
+Register map (v = VGPR, a = AGPR, s = SGPR):
+  a[32i+4o : +3]   accumulator of row block i, operand o = 2j+h (16-column group j, half h)
+  v[32b+4o : +3]   unpacked weights, buffer b (k step parity), operand o
+  v[64+4x : +3]    activation operand ring, x = row block % 4
+  v[80+4i : +3]    activation slab staging register i (8 per thread)
+  v[112+16u+4r:+3] packed weights of stage parity u, 16-deep row r of the stage
+  v[144+4u : +3]   group scales of stage parity u
+  v[152+i]         byte offset of this thread's row i in A (or the out-of-range flag)
+  v160 v161        per-lane byte offsets into B and into the scale rows
+  v162 v163        LDS addresses: operand reads, slab writes
+  v164 v165        shifted words of the unpack;  v166 0x64006400;  v167 -72 (fp16 x2)
+  v168             LDS address for the accumulators that go to the other k half
+  s[40:43] s[44:47] s[48:51]   buffer resources of A (tile rows), B, scales
+  s52 s53 s54      first stage, end stage of this k half; stages the loop runs
+  s55 s56          bytes per packed row of B; bytes per scale row
+  s57..s67         loop state and constants (see below)
+"""
+import sys
+
+RB = 8
+PLANE = 128 * 16
+STEP_BYTES = 4 * PLANE + 128
+SLAB_BYTES = 2 * STEP_BYTES           # 16640 = 65 * 256
+assert SLAB_BYTES % 256 == 0
+
+
+def W(b, o): return 32 * b + 4 * o
+def AF(x): return 64 + 4 * x
+def AREG(i): return 80 + 4 * i
+def BQ(u, r): return 112 + 16 * u + 4 * r
+def SREG(u): return 144 + 4 * u
+def ALANE(i): return 152 + i
+VBOFF, VSOFF, VRD, VWR = 160, 161, 162, 163
+WT = (164, 165)
+VEX, VNEG72, VSWAP = 166, 167, 168
+N_VGPR = 169
+RA, RB_, RS = 40, 44, 48
+S_BEGIN, S_END, S_STAGES, S_BROW, S_N2 = 52, 53, 54, 55, 56
+S_CS, S_SG2, S_SOFFA, S_SOFFB, S_SOFFS, S_FULL = 57, 58, 59, 60, 61, 62
+S_LOMASK, S_HIMASK, S_NEG1032, S_SIXTEENTH, S_TMP = 63, 64, 65, 66, 67
+
+
+def q(base): return f"v[{base}:{base + 3}]"
+def aq(base): return f"a[{base}:{base + 3}]"
+def sq(base): return f"s[{base}:{base + 3}]"
+
+
+class Emitter:
+    """Collects instructions and works out the s_waitcnt immediates.
+
+    Loads and LDS operations complete in order of issue, each kind on its own
+    counter.  wait_vm(reg) / wait_lgkm(reg) emit a wait that lets exactly the
+    operations issued after the one that last wrote `reg` stay in flight.  The
+    loop body is generated twice by the caller; only the second copy is kept,
+    so that producers in the previous turn are counted right."""
+
+    def __init__(self):
+        self.lines = []
+        self.vm = []      # destination base registers of loads, in issue order
+        self.lgkm = []    # destination base register (reads) or None (writes)
+
+    def emit(self, text):
+        self.lines.append(text)
+
+    def load(self, dst, voff, rsrc, soff):
+        self.emit(f"buffer_load_dwordx4 {q(dst)}, v{voff}, {sq(rsrc)}, s{soff} offen")
+        self.vm.append(dst)
+
+    def lds_read(self, dst, off):
+        assert 0 <= off < 65536
+        self.emit(f"ds_read_b128 {q(dst)}, v{VRD} offset:{off}")
+        self.lgkm.append(dst)
+
+    def lds_write2(self, d0, d1, off0, off1):
+        assert 0 <= off0 < 256 and 0 <= off1 < 256
+        self.emit(f"ds_write2st64_b32 v{VWR}, v{d0}, v{d1} offset0:{off0} offset1:{off1}")
+        self.lgkm.append(None)
+
+    @staticmethod
+    def _pending_after(queue, reg):
+        for back, r in enumerate(reversed(queue)):
+            if r == reg:
+                return back
+        return None  # written before anything tracked: it has landed
+
+    def wait(self, vm_regs=(), lgkm_regs=()):
+        vm = min([n for n in (self._pending_after(self.vm, r) for r in vm_regs) if n is not None],
+                 default=None)
+        lg = min([n for n in (self._pending_after(self.lgkm, r) for r in lgkm_regs)
+                  if n is not None], default=None)
+        parts = []
+        if vm is not None:
+            parts.append(f"vmcnt({min(vm, 63)})")
+        if lg is not None:
+            parts.append(f"lgkmcnt({min(lg, 15)})")
+        if parts:
+            self.emit("s_waitcnt " + " ".join(parts))
+
+    def drained(self, vm=False, lgkm=False):
+        """everything of that kind has completed (after an s_waitcnt ...(0))"""
+        if vm:
+            self.vm = []
+        if lgkm:
+            self.lgkm = []
+
+
+def unpack_ops(e, group, buf, u, rows, j, op):
+    """operation `op` of the unpack of word j of the two packed rows `rows` of
+    stage parity u into operands 2j, 2j+1 of buffer buf (both rows in lockstep)"""
+    for r in (0, 1):
+        src = BQ(u, rows[r]) + j
+        lo, hi = W(buf, 2 * j), W(buf, 2 * j + 1)
+        wt = WT[r]
+        if op == 0:
+            e.emit(f"v_lshrrev_b32 v{wt}, 8, v{src}")
+        elif op == 1:
+            e.emit(f"v_and_or_b32 v{lo + 2 * r}, v{src}, s{S_LOMASK}, v{VEX}")
+        elif op == 2:
+            e.emit(f"v_and_or_b32 v{lo + 2 * r + 1}, v{src}, s{S_HIMASK}, v{VEX}")
+        elif op == 3:
+            e.emit(f"v_and_or_b32 v{hi + 2 * r}, v{wt}, s{S_LOMASK}, v{VEX}")
+        elif op == 4:
+            e.emit(f"v_and_or_b32 v{hi + 2 * r + 1}, v{wt}, s{S_HIMASK}, v{VEX}")
+        elif op in (5, 7):
+            d = (lo if op == 5 else hi) + 2 * r
+            e.emit(f"v_pk_add_f16 v{d}, v{d}, s{S_NEG1032} op_sel_hi:[1,0]")
+        elif op in (6, 8):
+            d = (lo if op == 6 else hi) + 2 * r + 1
+            e.emit(f"v_pk_fma_f16 v{d}, v{d}, s{S_SIXTEENTH}, v{VNEG72} op_sel_hi:[1,0,0]")
+        else:
+            assert group
+            sc = SREG(u) + j
+            if op in (9, 10):    # columns c: the scale in the low half
+                d = lo + 2 * r + (op - 9)
+                e.emit(f"v_pk_mul_f16 v{d}, v{sc}, v{d} op_sel_hi:[0,1]")
+            else:                # columns c+8: the scale in the high half
+                d = hi + 2 * r + (op - 11)
+                e.emit(f"v_pk_mul_f16 v{d}, v{sc}, v{d} op_sel:[1,0] op_sel_hi:[1,1]")
+
+
+def stage_scalars(e, ahead):
+    """SALU: validity and offsets of the stage `ahead` stages after s57"""
+    e.emit(f"s_add_i32 s{S_SG2}, s{S_CS}, {ahead}")
+    e.emit(f"s_add_i32 s{S_SG2}, s{S_SG2}, s{S_BEGIN}")
+    # a stage past the end of this k half reads zeros for A: empty buffer
+    e.emit(f"s_cmp_lt_i32 s{S_SG2}, s{S_END}")
+    e.emit(f"s_cselect_b32 s{RA + 2}, s{S_FULL}, 0")
+    e.emit(f"s_lshl_b32 s{S_SOFFA}, s{S_SG2}, 7")
+    e.emit(f"s_lshl_b32 s{S_TMP}, s{S_SG2}, 2")
+    e.emit(f"s_mul_i32 s{S_SOFFB}, s{S_TMP}, s{S_BROW}")
+    e.emit(f"s_lshr_b32 s{S_TMP}, s{S_SG2}, 1")
+    e.emit(f"s_mul_i32 s{S_SOFFS}, s{S_TMP}, s{S_N2}")
+
+
+def load_b(e, u, r):
+    """row r of the stage that stage_scalars addressed (rows in order 0..3)"""
+    e.load(BQ(u, r), VBOFF, RB_, S_SOFFB)
+    e.emit(f"s_add_i32 s{S_SOFFB}, s{S_SOFFB}, s{S_BROW}")
+
+
+def slab_op(e, slab, x, first_i):
+    """x-th of the 12 slab operations of a step: per staging register two
+    ds_write2st64_b32 into LDS slab `slab`, then its reload for the stage that
+    stage_scalars addressed"""
+    i, g = first_i + x // 3, x % 3
+    if g < 2:
+        if g == 0:
+            e.wait(vm_regs=[AREG(i)])
+        unit = slab * (SLAB_BYTES // 256) + 16 * g + i
+        e.lds_write2(AREG(i) + 2 * g, AREG(i) + 2 * g + 1, unit, unit + 8)
+    else:
+        e.load(AREG(i), ALANE(i), RA, S_SOFFA)
+
+
+def mfma(e, i, o, buf, x):
+    acc = 32 * i + 4 * o
+    e.emit(f"v_mfma_f32_16x16x32_f16 {aq(acc)}, {q(W(buf, o))}, {q(AF(x))}, {aq(acc)}")
+
+
+def step(e, group, h, u, slab_cur, extra, unpack_rows_u, unpack_rows):
+    """64 MFMAs on buffer h and LDS step (slab_cur, h); the unpack of the next
+    step into buffer h^1; extra(m) issues memory operations behind MFMA m"""
+    ops_per_word = 13 if group else 9
+    cur = slab_cur * SLAB_BYTES + h * STEP_BYTES
+    nxt = (slab_cur * SLAB_BYTES + STEP_BYTES) if h == 0 else (slab_cur ^ 1) * SLAB_BYTES
+    for i in range(RB):
+        tgt = i + 3
+        e.lds_read(AF(tgt & 3), (cur + tgt * 256) if tgt < RB else (nxt + (tgt - RB) * 256))
+        e.wait(lgkm_regs=[AF(i & 3)])
+        for o in range(8):
+            m = 8 * i + o
+            mfma(e, i, o, h, i & 3)
+            if m == 0:
+                # the packed rows (and scales) of the step being unpacked
+                regs = [BQ(unpack_rows_u, unpack_rows[0]), BQ(unpack_rows_u, unpack_rows[1])]
+                if group:
+                    regs.append(SREG(unpack_rows_u))
+                e.wait(vm_regs=regs)
+            if m < 4 * ops_per_word:
+                unpack_ops(e, group, h ^ 1, unpack_rows_u, unpack_rows, m // ops_per_word,
+                           m % ops_per_word)
+            extra(m)
+
+
+def stage(e, group, u):
+    """One 64-deep stage cs of parity u.  Step 0: rows 2, 3 of this stage are
+    unpacked, staging registers 0..3 go to LDS slab u^1 (stage cs+1) and are
+    requested again for stage cs+2, rows 0, 1 of stage cs+2 are requested.
+    Step 1: rows 0, 1 of stage cs+1 are unpacked, staging registers 4..7 go to
+    LDS; then the one barrier of the stage -- after it nobody reads slab u
+    again, so the next stage may overwrite it, and slab u^1 is complete --
+    before the first operands of stage cs+1 are read; rows 2, 3 and the scales
+    of stage cs+2 are requested."""
+    stage_scalars(e, 2 + u)  # s57 counts the turn's first stage
+
+    def extra0(m):
+        if m % 4 == 2 and m // 4 < 12:
+            slab_op(e, u ^ 1, m // 4, 0)
+        if m == 50:
+            load_b(e, u, 0)
+        if m == 54:
+            load_b(e, u, 1)
+
+    def extra1(m):
+        if m % 3 == 1 and m // 3 < 12:
+            slab_op(e, u ^ 1, m // 3, 4)
+        if m == 37:
+            e.emit("s_waitcnt lgkmcnt(0)")
+            e.drained(lgkm=True)
+            e.emit("s_barrier")
+        if m == 42:
+            load_b(e, u, 2)
+        if m == 46:
+            load_b(e, u, 3)
+        if m == 50 and group:
+            e.load(SREG(u), VSOFF, RS, S_SOFFS)
+
+    step(e, group, 0, u, u, extra0, u, (2, 3))
+    step(e, group, 1, u, u, extra1, u ^ 1, (0, 1))
+
+
+def prologue(e, group):
+    e.emit(f"s_mov_b32 s{S_FULL}, s{RA + 2}")
+    e.emit(f"s_mov_b32 s{S_CS}, 0")
+    e.emit(f"s_mov_b32 s{S_LOMASK}, 0x000f000f")
+    e.emit(f"s_mov_b32 s{S_HIMASK}, 0x00f000f0")
+    e.emit(f"s_mov_b32 s{S_NEG1032}, 0xe408")      # fp16 -1032
+    e.emit(f"s_mov_b32 s{S_SIXTEENTH}, 0x2c00")    # fp16 1/16
+    e.emit(f"v_mov_b32 v{VEX}, 0x64006400")
+    e.emit(f"v_mov_b32 v{VNEG72}, 0xd480")         # fp16 -72
+    for st in (0, 1):
+        stage_scalars(e, st)
+        for r in range(4):
+            load_b(e, st, r)
+        if group:
+            e.load(SREG(st), VSOFF, RS, S_SOFFS)
+        if st == 0:
+            for i in range(RB):
+                e.load(AREG(i), ALANE(i), RA, S_SOFFA)
+            # the accumulators start at zero
+            for n in range(256):
+                e.emit(f"v_accvgpr_write_b32 a{n}, 0")
+        else:
+            # slab 0 to LDS, its registers requested again for stage 1
+            for i in range(RB):
+                for x in range(3):
+                    slab_op(e, 0, 3 * i + x, 0)
+    # first k step's weights
+    regs = [BQ(0, 0), BQ(0, 1)] + ([SREG(0)] if group else [])
+    e.wait(vm_regs=regs)
+    for j in range(4):
+        for op in range(13 if group else 9):
+            unpack_ops(e, group, 0, 0, (0, 1), j, op)
+    # everything requested so far has landed before the loop starts, so that
+    # the loop's waits, computed for its steady state, hold in its first turn
+    e.emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    e.drained(vm=True, lgkm=True)
+    e.emit("s_barrier")
+    for x in range(3):
+        e.lds_read(AF(x), x * 256)
+
+
+def epilogue(e):
+    # the last MFMAs' results are not readable for 18 cycles, and the hardware
+    # does not interlock that for what follows
+    e.emit("s_nop 15")
+    e.emit("s_nop 15")
+    e.emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    e.emit("s_barrier")          # every wave is done with the slabs
+    for i in range(4, RB):
+        for o in range(8):
+            e.emit(f"ds_write_b128 v{VSWAP}, {aq(32 * i + 4 * o)} offset:{((i - 4) * 8 + o) * 1024}")
+    for n in range(128):
+        e.emit(f"v_accvgpr_read_b32 v{n}, a{n}")
+    e.emit("s_waitcnt lgkmcnt(0)")
+
+
+def generate(group):
+    e = Emitter()
+    prologue(e, group)
+    head = len(e.lines)
+    # the loop body twice: the first copy only sets up the issue history
+    for copy in (0, 1):
+        if copy == 1:
+            body_start = len(e.lines)
+        e.emit(".Lwd_loop_%=:")
+        stage(e, group, 0)
+        e.emit(f"s_add_i32 s{S_TMP}, s{S_CS}, 1")
+        e.emit(f"s_cmp_ge_i32 s{S_TMP}, s{S_STAGES}")
+        e.emit("s_cbranch_scc1 .Lwd_done_%=")
+        stage(e, group, 1)
+        e.emit(f"s_add_i32 s{S_CS}, s{S_CS}, 2")
+        e.emit(f"s_cmp_lt_i32 s{S_CS}, s{S_STAGES}")
+        e.emit("s_cbranch_scc1 .Lwd_loop_%=")
+    lines = e.lines[:head] + e.lines[body_start:]
+    e.lines = []
+    e.emit(".Lwd_done_%=:")
+    epilogue(e)
+    lines += e.lines
+    return lines
+
+
+def statement(group):
+    lines = generate(group)
+    out = ["// generated by gen_prefill_wide.py -- do not edit", "asm volatile("]
+    out += [f'    "{l}\\n\\t"' for l in lines]
+    outs = [f'"={{v[{32 * i + 4 * o}:{32 * i + 4 * o + 3}]}}"(fin[{i}][{o}])'
+            for i in range(4) for o in range(8)]
+    outs.append(f'"+{{s[{RA}:{RA + 3}]}}"(ra_words)')
+    out.append("    : " + ",\n      ".join(outs))
+    ins = [f'"{{s[{RB_}:{RB_ + 3}]}}"(rb_words)',
+           f'"{{s[{RS}:{RS + 3}]}}"(rs_words)',
+           f'"{{s{S_BEGIN}}}"(s_begin)', f'"{{s{S_END}}}"(s_end)', f'"{{s{S_STAGES}}}"(stages)',
+           f'"{{s{S_BROW}}}"(b_row)', f'"{{s{S_N2}}}"(s_row)']
+    ins += [f'"{{v{ALANE(i)}}}"(a_lane[{i}])' for i in range(RB)]
+    ins += [f'"{{v{VBOFF}}}"(b_lane)', f'"{{v{VSOFF}}}"(s_lane)', f'"{{v{VRD}}}"(lds_rd)',
+            f'"{{v{VWR}}}"(lds_wr)', f'"{{v{VSWAP}}}"(lds_swap)']
+    out.append("    : " + ",\n      ".join(ins))
+    clob = [f'"v{n}"' for n in range(128, 152)] + [f'"v{n}"' for n in (164, 165, 166, 167)]
+    clob += [f'"a{n}"' for n in range(256)]
+    clob += [f'"s{n}"' for n in range(S_CS, S_TMP + 1)] + ['"scc"', '"memory"']
+    out.append("    : " + ", ".join(clob) + ");")
+    return "\n".join(out) + "\n"
+
+
+if __name__ == "__main__":
+    outdir = sys.argv[1] if len(sys.argv) > 1 else "."
+    for group, name in ((True, "group"), (False, "chan")):
+        with open(f"{outdir}/w4a16_prefill_wide_{name}.inc", "w") as f:
+            f.write(statement(group))

@@ -186,6 +186,9 @@ int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 // counter per tile, zero again afterwards)
 // tile_rows: rows of C per workgroup, 64 or 128
 int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream);
+// the 128-row tiles on four waves with 128 x 128 accumulators (w4a16_prefill_wide.hip)
+int configure_prefill_wide_kernels();
+int launch_prefill_wide(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
 
 // Measurement probes (w4a16_probe.hip): an empty launch of `grid` workgroups,
 // and a plain read of the packed weights with the streaming kernel's work split
