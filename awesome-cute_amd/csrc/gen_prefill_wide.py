@@ -34,6 +34,16 @@ Register map (v = VGPR, a = AGPR, s = SGPR):
 """
 import sys
 
+# Schedule knobs (key=value on the command line overrides; the defaults are
+# the measured best):
+#   ahead    row blocks between an operand's LDS read and its first MFMA (1..3)
+#   rdoff    MFMA of a row block behind which the read is issued (0..7)
+#   slab0    preferred first MFMA and stride of the 12 slab operations of step 0
+#   slab1    the same for step 1 (they end before the barrier, which sits just
+#            before the first operand read from the next slab)
+#   b0, b1   preferred MFMAs of the weight (and scale) loads of steps 0 and 1
+OPT = {"ahead": 2, "rdoff": 0, "slab0": (2, 5), "slab1": (1, 3.5), "b0": (52, 58), "b1": (52, 56, 60)}
+
 RB = 8
 PLANE = 128 * 16
 STEP_BYTES = 4 * PLANE + 128
@@ -121,10 +131,10 @@ class Emitter:
             self.lgkm = []
 
 
-def unpack_ops(e, group, buf, u, rows, j, op):
-    """operation `op` of the unpack of word j of the two packed rows `rows` of
-    stage parity u into operands 2j, 2j+1 of buffer buf (both rows in lockstep)"""
-    for r in (0, 1):
+def unpack_op(e, group, buf, u, rows, j, op, r):
+    """operation `op` of the unpack of word j of packed row rows[r] of stage
+    parity u into dwords 2r, 2r+1 of operands 2j, 2j+1 of buffer buf"""
+    if True:
         src = BQ(u, rows[r]) + j
         lo, hi = W(buf, 2 * j), W(buf, 2 * j + 1)
         wt = WT[r]
@@ -194,29 +204,79 @@ def mfma(e, i, o, buf, x):
     e.emit(f"v_mfma_f32_16x16x32_f16 {aq(acc)}, {q(W(buf, o))}, {q(AF(x))}, {aq(acc)}")
 
 
-def step(e, group, h, u, slab_cur, extra, unpack_rows_u, unpack_rows):
-    """64 MFMAs on buffer h and LDS step (slab_cur, h); the unpack of the next
-    step into buffer h^1; extra(m) issues memory operations behind MFMA m"""
+def assign_slots(prefs):
+    """distinct MFMA slots 0..63 for operations with preferred slots `prefs`
+    (ascending): each gets its preference or the next free slot after the one
+    before it; if they run past the end, the tail is pushed back"""
+    slots, last = [], -1
+    for pr in prefs:
+        last = max(last + 1, int(pr))
+        slots.append(last)
+    over = slots[-1] - 63 if slots else 0
+    if over > 0:
+        for k in range(len(slots) - 1, -1, -1):
+            cap = 63 - (len(slots) - 1 - k)
+            if slots[k] <= cap:
+                break
+            slots[k] = cap
+    assert len(set(slots)) == len(slots) and all(0 <= x < 64 for x in slots), slots
+    return slots
+
+
+def step(e, group, h, slab_cur, mem_ops, unpack_u, unpack_rows):
+    """64 MFMAs on buffer h and LDS step (slab_cur, h), while the next step's
+    weights (rows unpack_rows of stage parity unpack_u) are unpacked into buffer
+    h^1 and the memory operations mem_ops -- (preferred slot, emit function),
+    the step's operand reads are added here -- are issued.
+
+    A memory instruction and unpack arithmetic behind the same MFMA cost about
+    a whole MFMA time more than either alone (measured: MFMAs with the unpack
+    16.2 cycles per MFMA, with the memory operations 17.7, with both dealt out
+    regardless 23.0), so every memory operation gets an MFMA of its own, and
+    the unpack goes behind the others, two operations each and three where
+    that is not enough."""
     ops_per_word = 13 if group else 9
     cur = slab_cur * SLAB_BYTES + h * STEP_BYTES
     nxt = (slab_cur * SLAB_BYTES + STEP_BYTES) if h == 0 else (slab_cur ^ 1) * SLAB_BYTES
+    ahead = OPT["ahead"]
+    ops = list(mem_ops)
     for i in range(RB):
-        tgt = i + 3
-        e.lds_read(AF(tgt & 3), (cur + tgt * 256) if tgt < RB else (nxt + (tgt - RB) * 256))
+        tgt = i + ahead
+        off = (cur + tgt * 256) if tgt < RB else (nxt + (tgt - RB) * 256)
+        ops.append((8 * i + OPT["rdoff"], lambda e, tgt=tgt, off=off: e.lds_read(AF(tgt & 3), off)))
+    ops.sort(key=lambda x: x[0])
+    slots = assign_slots([pr for pr, _ in ops])
+    mem_at = dict(zip(slots, (fn for _, fn in ops)))
+    # the unpack: 8 words x ops_per_word operations, rows in lockstep
+    todo = [(t // ops_per_word, t % ops_per_word, r) for t in range(4 * ops_per_word)
+            for r in (0, 1)]
+    free = [m for m in range(64) if m not in mem_at]
+    per = [2] * len(free)
+    short = len(todo) - 2 * len(free)
+    k = 0
+    while short > 0:      # a third operation behind evenly spaced MFMAs
+        per[(k * len(free)) // max(1, len(todo) - 2 * len(free))] += 1
+        k += 1
+        short -= 1
+    valu_at = dict(zip(free, per))
+    for i in range(RB):
         e.wait(lgkm_regs=[AF(i & 3)])
         for o in range(8):
             m = 8 * i + o
             mfma(e, i, o, h, i & 3)
-            if m == 0:
+            if m in mem_at:
+                mem_at[m](e)
+            n = min(valu_at.get(m, 0), len(todo))
+            if n and len(todo) == 8 * ops_per_word:
                 # the packed rows (and scales) of the step being unpacked
-                regs = [BQ(unpack_rows_u, unpack_rows[0]), BQ(unpack_rows_u, unpack_rows[1])]
+                regs = [BQ(unpack_u, unpack_rows[0]), BQ(unpack_u, unpack_rows[1])]
                 if group:
-                    regs.append(SREG(unpack_rows_u))
+                    regs.append(SREG(unpack_u))
                 e.wait(vm_regs=regs)
-            if m < 4 * ops_per_word:
-                unpack_ops(e, group, h ^ 1, unpack_rows_u, unpack_rows, m // ops_per_word,
-                           m % ops_per_word)
-            extra(m)
+            for _ in range(n):
+                j, op, r = todo.pop(0)
+                unpack_op(e, group, h ^ 1, unpack_u, unpack_rows, j, op, r)
+    assert not todo
 
 
 def stage(e, group, u):
@@ -230,30 +290,23 @@ def stage(e, group, u):
     of stage cs+2 are requested."""
     stage_scalars(e, 2 + u)  # s57 counts the turn's first stage
 
-    def extra0(m):
-        if m % 4 == 2 and m // 4 < 12:
-            slab_op(e, u ^ 1, m // 4, 0)
-        if m == 50:
-            load_b(e, u, 0)
-        if m == 54:
-            load_b(e, u, 1)
+    def barrier(e):
+        e.emit("s_waitcnt lgkmcnt(0)")
+        e.drained(lgkm=True)
+        e.emit("s_barrier")
 
-    def extra1(m):
-        if m % 3 == 1 and m // 3 < 12:
-            slab_op(e, u ^ 1, m // 3, 4)
-        if m == 37:
-            e.emit("s_waitcnt lgkmcnt(0)")
-            e.drained(lgkm=True)
-            e.emit("s_barrier")
-        if m == 42:
-            load_b(e, u, 2)
-        if m == 46:
-            load_b(e, u, 3)
-        if m == 50 and group:
-            e.load(SREG(u), VSOFF, RS, S_SOFFS)
-
-    step(e, group, 0, u, u, extra0, u, (2, 3))
-    step(e, group, 1, u, u, extra1, u ^ 1, (0, 1))
+    a, st = OPT["slab0"]
+    ops0 = [(a + st * x, lambda e, x=x: slab_op(e, u ^ 1, x, 0)) for x in range(12)]
+    ops0 += [(OPT["b0"][r], lambda e, r=r: load_b(e, u, r)) for r in (0, 1)]
+    a, st = OPT["slab1"]
+    bar = 8 * (RB - OPT["ahead"]) + OPT["rdoff"] - 0.5  # just before the first read of the next slab
+    ops1 = [(min(a + st * x, bar - 0.75), lambda e, x=x: slab_op(e, u ^ 1, x, 4)) for x in range(12)]
+    ops1 += [(bar, barrier)]
+    ops1 += [(OPT["b1"][r], lambda e, r=r: load_b(e, u, 2 + r)) for r in (0, 1)]
+    if group:
+        ops1 += [(OPT["b1"][2], lambda e: e.load(SREG(u), VSOFF, RS, S_SOFFS))]
+    step(e, group, 0, u, ops0, u, (2, 3))
+    step(e, group, 1, u, ops1, u ^ 1, (0, 1))
 
 
 def prologue(e, group):
@@ -287,13 +340,14 @@ def prologue(e, group):
     e.wait(vm_regs=regs)
     for j in range(4):
         for op in range(13 if group else 9):
-            unpack_ops(e, group, 0, 0, (0, 1), j, op)
+            for r in (0, 1):
+                unpack_op(e, group, 0, 0, (0, 1), j, op, r)
     # everything requested so far has landed before the loop starts, so that
     # the loop's waits, computed for its steady state, hold in its first turn
     e.emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e.drained(vm=True, lgkm=True)
     e.emit("s_barrier")
-    for x in range(3):
+    for x in range(OPT["ahead"]):
         e.lds_read(AF(x), x * 256)
 
 
@@ -362,6 +416,9 @@ def statement(group):
 
 if __name__ == "__main__":
     outdir = sys.argv[1] if len(sys.argv) > 1 else "."
+    for arg in sys.argv[2:]:
+        key, val = arg.split("=")
+        OPT[key] = tuple(float(x) for x in val.split(",")) if "," in val else int(val)
     for group, name in ((True, "group"), (False, "chan")):
         with open(f"{outdir}/w4a16_prefill_wide_{name}.inc", "w") as f:
             f.write(statement(group))
