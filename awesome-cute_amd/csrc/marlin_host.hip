@@ -121,7 +121,6 @@ struct Plan {
   int launches;
   int ksplit;            // prefill: slices of the k range per tile
   int tile_rows;         // prefill: rows of C per workgroup
-  bool wide;             // prefill, 128 rows: the four-wave kernel
   size_t partial_bytes;  // fp32 partial sums the launch exchanges through scratch (0: none)
 };
 
@@ -206,7 +205,6 @@ double prefill_cost_rows(int m, int n, int k, const PlanCtx& cx, int tile_rows) 
 // 21.9 us), at N = 4096, K = 11008 up to 256 (27.5 against 38.9 us at M = 128).
 int prefill_tile_rows(int m, int n, int k, const PlanCtx& cx) {
   if (cx.force.tile_rows == 64 || cx.force.tile_rows == 128) return cx.force.tile_rows;
-  if (cx.force.tile_rows == 130) return 128;
   if (m <= 64) return 64;
   return prefill_cost_rows(m, n, k, cx, 64) < prefill_cost_rows(m, n, k, cx, 128) ? 64 : 128;
 }
@@ -296,20 +294,14 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   const bool prefill =
       n % 256 == 0 && (force == 2 || (force == 0 && prefer_prefill(m, n, k, cx)));
   pl.ksplit = 1;
-  pl.wide = false;
   pl.tile_rows = 0;
   pl.partial_bytes = 0;
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
     pl.tile_rows = prefill_tile_rows(m, n, k, cx);
-    pl.wide = false;
-    const int tiles = ceil_div(m, pl.tile_rows) * (n / 256);
+      const int tiles = ceil_div(m, pl.tile_rows) * (n / 256);
     pl.ksplit = prefill_k_slices(tiles, pl.tile_rows, k, cx);
-    // 128-row tiles: the four-wave kernel where the k range is not sliced
-    // (2-4 % faster there, 1-4 % slower with slices)
-    pl.wide = pl.tile_rows == 128 &&
-              (cx.force.tile_rows == 130 || (cx.force.tile_rows == 0 && pl.ksplit == 1));
     pl.grid = tiles * pl.ksplit;
     pl.sp = make_stream_plan(n, k, 1);
     pl.launches = 1;
@@ -365,8 +357,10 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
     a.scratch = view.partials;
     a.gpb = 0;
     a.wpt = 0;
-    rc = pl.wide ? launch_prefill_wide(a, groupsize != -1, pl.ksplit, stream)
-                 : launch_prefill(a, groupsize != -1, pl.ksplit, pl.tile_rows, stream);
+    // 128-row tiles: four waves with 128 x 128 accumulators; 64-row tiles: eight
+    // waves with 64 x 64
+    rc = pl.tile_rows == 128 ? launch_prefill_wide(a, groupsize != -1, pl.ksplit, stream)
+                             : launch_prefill(a, groupsize != -1, pl.ksplit, stream);
   } else {
     for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
       GemmArgs a;
@@ -575,9 +569,7 @@ void marlin_amd_force_kernel(int which) { t_force.kernel = which == 1 || which =
 
 void marlin_amd_force_k_slices(int slices) { t_force.k_slices = slices > 0 ? slices : 0; }
 
-void marlin_amd_force_tile_rows(int rows) {
-  t_force.tile_rows = rows == 64 || rows == 128 || rows == 130 ? rows : 0;
-}
+void marlin_amd_force_tile_rows(int rows) { t_force.tile_rows = rows == 64 || rows == 128 ? rows : 0; }
 
 void marlin_amd_work_order(int grid, int* out) {
   for (int b = 0; b < grid; b++) out[b] = xcd_work_index(b, grid);

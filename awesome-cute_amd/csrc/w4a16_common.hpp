@@ -184,9 +184,10 @@ int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 // ksplit >= 1 slices of the k range per tile; above 1 the launch needs
 // a.scratch (ksplit * tiles * tile bytes of fp32) and a.locks (one zeroed
 // counter per tile, zero again afterwards)
-// tile_rows: rows of C per workgroup, 64 or 128
-int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream);
-// the 128-row tiles on four waves with 128 x 128 accumulators (w4a16_prefill_wide.hip)
+// 64-row x 256-column tiles, eight waves (w4a16_prefill.hip)
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
+// 128-row x 256-column tiles, four waves with 128 x 128 accumulators
+// (w4a16_prefill_wide.hip); same scratch layout and counters
 int configure_prefill_wide_kernels();
 int launch_prefill_wide(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
 

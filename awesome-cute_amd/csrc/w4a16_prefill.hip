@@ -558,7 +558,7 @@ static int configure_rb() {
   return 0;
 }
 
-int configure_prefill_kernels() { return (configure_rb<8>() | configure_rb<4>()) ? 3 : 0; }
+int configure_prefill_kernels() { return configure_rb<4>() ? 3 : 0; }
 
 template <bool GROUP, int RB>
 static void launch_rb(const GemmArgs& a, int ksplit, hipStream_t stream) {
@@ -569,12 +569,8 @@ static void launch_rb(const GemmArgs& a, int ksplit, hipStream_t stream) {
                      stream, a, tiles_m, tiles_n, ksplit);
 }
 
-int launch_prefill(const GemmArgs& a, bool group, int ksplit, int tile_rows, hipStream_t stream) {
-  if (tile_rows == 64) {
-    if (group) launch_rb<true, 4>(a, ksplit, stream); else launch_rb<false, 4>(a, ksplit, stream);
-  } else {
-    if (group) launch_rb<true, 8>(a, ksplit, stream); else launch_rb<false, 8>(a, ksplit, stream);
-  }
+int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream) {
+  if (group) launch_rb<true, 4>(a, ksplit, stream); else launch_rb<false, 4>(a, ksplit, stream);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
