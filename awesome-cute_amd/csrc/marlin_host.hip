@@ -25,6 +25,13 @@ constexpr size_t kStaticPartialBytes = (size_t)32 << 20;
 constexpr size_t kStaticScratchBytes = w4a16::kCounterBytes + kStaticPartialBytes;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
+namespace w4a16 {
+hipError_t& last_launch_error() {
+  thread_local hipError_t e = hipSuccess;
+  return e;
+}
+}  // namespace w4a16
+
 namespace {
 
 using namespace w4a16;
@@ -36,12 +43,6 @@ thread_local char g_last_error[256] = "";
 
 void set_error(hipError_t e, const char* what) {
   snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
-}
-
-// A fill kernel rather than a memset, so that it may be recorded into a graph.
-__global__ void scratch_clear_kernel(int* p, int count) {
-  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
-  if (i < count) p[i] = 0;
 }
 
 struct DeviceState {
@@ -379,14 +380,15 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
       rc = launch_stream(a, groupsize != -1, pl.grid, stream);
     }
   }
-  if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "kernel launch");
+  if (rc == MARLIN_ERR_RUNTIME) set_error(w4a16::last_launch_error(), "kernel launch");
   return rc;
 }
 
-// With `dev` current: this device's copy of the fixed scratch array, its
-// counters cleared once (on `stream`, by a kernel, so that a first call under
-// capture records the clearing like any other node).
-unsigned char* static_scratch_for(int dev, hipStream_t stream) {
+// With `dev` current: this device's copy of the fixed scratch array.  Its
+// counters need no clearing: the array is zero when the module is loaded and
+// every launch hands its counters back zeroed.  (A clearing kernel on the first
+// caller's stream could land in the middle of another stream's first launch.)
+unsigned char* static_scratch_for(int dev) {
   std::lock_guard<std::mutex> lk(g_mu);
   DeviceState& d = g_dev[dev];
   if (d.static_scratch) return d.static_scratch;
@@ -394,13 +396,6 @@ unsigned char* static_scratch_for(int dev, hipStream_t stream) {
   hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
   if (e != hipSuccess || !ptr) {
     set_error(e, "hipGetSymbolAddress(scratch)");
-    return nullptr;
-  }
-  hipLaunchKernelGGL(scratch_clear_kernel, dim3(kMaxCounters / 256), dim3(256), 0, stream,
-                     (int*)ptr, kMaxCounters);
-  e = hipGetLastError();
-  if (e != hipSuccess) {
-    set_error(e, "scratch_clear_kernel");
     return nullptr;
   }
   d.static_scratch = (unsigned char*)ptr;
@@ -455,7 +450,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
                  m, n, k, sms, pl.partial_bytes, kStaticPartialBytes);
         ok = false;
       } else if (pl.partial_bytes > 0) {
-        unsigned char* base = static_scratch_for(dev, stream);
+        unsigned char* base = static_scratch_for(dev);
         ok = base != nullptr;
         if (ok) {
           view.counters = (int*)base;
@@ -602,25 +597,40 @@ int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, v
   int tk = -1, tn = -1;
   int rc = check_shape(1, prob_n, prob_k, -1, tk, tn);
   if (rc != MARLIN_OK) return rc;
-  if (prob_n == 0 || prob_k == 0 || dev < 0 || dev >= kMaxDevices) return MARLIN_ERR_PROB_SHAPE;
-  const int cus = device_cus(dev);
-  if (cus <= 0) return MARLIN_ERR_RUNTIME;
-  const PlanCtx cx = {cus, kPoolPartialLimit, Force()};
-  const Plan pl = make_plan(1, prob_n, prob_k, -1, cx);
-  (void)hipGetLastError();
-  if (kind == 0) {
-    rc = launch_probe_empty(pl.grid, stream);
-  } else {
-    GemmArgs a = {};
-    a.B = B;
-    a.M = 1;
-    a.N = prob_n;
-    a.K = prob_k;
-    a.gpb = pl.sp.gpb;
-    a.wpt = pl.sp.wpt;
-    rc = launch_probe_read(a, pl.grid, stream);
+  if (prob_n == 0 || prob_k == 0 || dev < 0 || dev >= kMaxDevices || kind < 0 || kind > 2)
+    return MARLIN_ERR_PROB_SHAPE;
+  int prev = -1;
+  hipError_t e = hipGetDevice(&prev);
+  if (e == hipSuccess && prev != dev) e = hipSetDevice(dev);
+  if (e != hipSuccess) {
+    set_error(e, "hipSetDevice");
+    return MARLIN_ERR_RUNTIME;
   }
-  if (rc == MARLIN_ERR_RUNTIME) set_error(hipGetLastError(), "probe launch");
+  const int cus = device_cus(dev);
+  rc = MARLIN_ERR_RUNTIME;
+  if (cus > 0) {
+    const PlanCtx cx = {cus, kPoolPartialLimit, Force()};
+    const Plan pl = make_plan(1, prob_n, prob_k, -1, cx);
+    (void)hipGetLastError();
+    if (kind == 0) {
+      rc = launch_probe_empty(pl.grid, stream);
+    } else if (kind == 1) {
+      GemmArgs a = {};
+      a.B = B;
+      a.M = 1;
+      a.N = prob_n;
+      a.K = prob_k;
+      a.gpb = pl.sp.gpb;
+      a.wpt = pl.sp.wpt;
+      rc = launch_probe_read(a, pl.grid, stream);
+    } else {
+      // one workgroup of 8 waves per CU; n*k/8192 MFMAs per wave (a multiple of 32)
+      const long long per_wave = (long long)prob_n * prob_k / 8192;
+      rc = launch_probe_mfma(cus, (int)(per_wave / 32 > 0 ? per_wave / 32 : 1), stream);
+    }
+    if (rc == MARLIN_ERR_RUNTIME) set_error(w4a16::last_launch_error(), "probe launch");
+  }
+  if (prev != dev) (void)hipSetDevice(prev);
   return rc;
 }
 

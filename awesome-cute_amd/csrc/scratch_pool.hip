@@ -81,21 +81,38 @@ bool scratch_acquire(int dev, hipStream_t stream, size_t partial_bytes, ScratchV
                  partial_bytes + kCounterBytes);
       return false;
     }
+    // buffers are keyed by stream handle and kept until scratch_release (a
+    // launch in flight or a captured graph may still name them), so a process
+    // that keeps making streams would grow without bound: refuse beyond a cap
+    if (g_buffers[dev].size() >= kPoolMaxBuffers) {
+      if (err && err_len)
+        snprintf(err, err_len,
+                 "%zu scratch buffers are held on device %d (one per stream that shared tiles, "
+                 "plus outgrown ones): call marlin_amd_release(%d) when those streams are idle",
+                 g_buffers[dev].size(), dev, dev);
+      return false;
+    }
     size_t want = (partial_bytes + kGrain - 1) / kGrain * kGrain;
     if (live && want < 2 * live->partial_bytes) want = 2 * live->partial_bytes;
     if (want < kGrain) want = kGrain;
+    // Another stream of this process may be under capture in the default
+    // (global) mode, in which an allocation from any thread invalidates that
+    // capture: this thread's calls below are made in relaxed mode.
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
     char* p = nullptr;
     e = hipMalloc((void**)&p, kCounterBytes + want);
+    // Cleared on the caller's stream, ahead of the launch that will use the
+    // counters: a clear on the null stream is not ordered against a
+    // non-blocking stream and could land in the middle of that launch.
+    hipError_t e2 = e == hipSuccess ? hipMemsetAsync(p, 0, kCounterBytes, stream) : hipSuccess;
+    if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
     if (e != hipSuccess) {
       fail(err, err_len, "hipMalloc(scratch)", e);
       return false;
     }
-    // Cleared on the caller's stream, ahead of the launch that will use the
-    // counters: a clear on the null stream is not ordered against a
-    // non-blocking stream and could land in the middle of that launch.
-    e = hipMemsetAsync(p, 0, kCounterBytes, stream);
-    if (e != hipSuccess) {
-      fail(err, err_len, "hipMemsetAsync(scratch)", e);
+    if (e2 != hipSuccess) {
+      fail(err, err_len, "hipMemsetAsync(scratch)", e2);
       (void)hipFree(p);
       return false;
     }

@@ -16,6 +16,9 @@ namespace w4a16 {
 constexpr size_t kCounterBytes = 64 * 1024;  // 16384 tile counters
 constexpr int kMaxCounters = (int)(kCounterBytes / sizeof(int));
 constexpr int kPoolMaxDevices = 16;
+// buffers held per device at most (live and outgrown ones together); every
+// stream handle that ever shared tiles keeps its buffer until scratch_release
+constexpr size_t kPoolMaxBuffers = 256;
 
 struct ScratchView {
   int* counters;    // kMaxCounters ints, zero between launches
@@ -25,8 +28,11 @@ struct ScratchView {
 // The scratch of (dev, stream) with room for partial_bytes of partial sums;
 // `dev` must be the current device.  Allocates or grows when needed: growing
 // waits for the stream's earlier work (which may still use the old buffer).
-// Fails -- returns false with a message in err -- when hipMalloc fails or when
-// an allocation would be needed while the stream is being captured into a graph.
+// Fails -- returns false with a message in err -- when hipMalloc fails, when
+// an allocation would be needed while the stream is being captured into a
+// graph, or when the device already holds kPoolMaxBuffers buffers.  (While
+// another stream is under capture the allocation is made in relaxed capture
+// mode, which leaves that capture valid.)
 bool scratch_acquire(int dev, hipStream_t stream, size_t partial_bytes, ScratchView* out,
                      char* err, size_t err_len);
 

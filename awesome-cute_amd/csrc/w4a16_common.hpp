@@ -175,6 +175,16 @@ struct GemmArgs {
 // bytes of fp32 partial sums of mb row blocks of 16 (one slot)
 constexpr size_t stream_slot_bytes(int mb) { return (size_t)mb * 4 * 2 * 64 * 16; }
 
+// Result of a kernel launch for the launch helpers below: 0, or 3 with the
+// runtime's error kept per thread for the caller's message (reading the
+// runtime's error state clears it, so the helper that reads it must keep it).
+hipError_t& last_launch_error();
+inline int launch_status() {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) last_launch_error() = e;
+  return e == hipSuccess ? 0 : 3;
+}
+
 // Per-device set-up of the kernels that need more dynamic LDS than the default
 // limit; call once with the device current before the first launch on it.
 int configure_stream_kernels();
@@ -196,5 +206,8 @@ int launch_prefill_wide(const GemmArgs& a, bool group, int ksplit, hipStream_t s
 // (a.B, a.N, a.K, a.gpb, a.wpt) and access pattern, no arithmetic.
 int launch_probe_empty(int grid, hipStream_t stream);
 int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream);
+// ... and a loop of nothing but MFMAs: grid workgroups of 8 waves, 32 * iters
+// v_mfma_f32_16x16x32_f16 per wave
+int launch_probe_mfma(int grid, int iters, hipStream_t stream);
 
 }  // namespace w4a16

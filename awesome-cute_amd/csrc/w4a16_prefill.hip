@@ -571,7 +571,7 @@ static void launch_rb(const GemmArgs& a, int ksplit, hipStream_t stream) {
 
 int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream) {
   if (group) launch_rb<true, 4>(a, ksplit, stream); else launch_rb<false, 4>(a, ksplit, stream);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  return launch_status();
 }
 
 }  // namespace w4a16

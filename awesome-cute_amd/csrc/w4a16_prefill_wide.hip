@@ -289,7 +289,7 @@ int launch_prefill_wide(const GemmArgs& a, bool group, int ksplit, hipStream_t s
   else
     hipLaunchKernelGGL(prefill_wide_kernel<false>, grid, dim3(256), kWdLdsBytes, stream, a,
                        tiles_m, tiles_n, ksplit);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  return launch_status();
 }
 
 }  // namespace w4a16

@@ -5,7 +5,10 @@
 // does for the same plan -- same work split, same workgroup-to-XCD order, same
 // 128-bit streaming buffer loads of 1 KiB per wave instruction, four rows per
 // granule -- keeps up to kProbeDepth granules in flight per wave, and throws
-// the data away.  probe_empty_kernel does nothing at all.
+// the data away.  probe_empty_kernel does nothing at all.  probe_mfma_kernel is
+// a loop of nothing but v_mfma_f32_16x16x32_f16 on pseudo-random operands, two
+// waves per SIMD and 32 independent accumulators per wave: what the matrix
+// pipes of this board sustain when nothing competes with them.
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
@@ -65,14 +68,56 @@ __global__ __launch_bounds__(256) void probe_read_kernel(GemmArgs p, int* sink) 
   if ((acc[0] & acc[1] & acc[2] & acc[3]) == 0x12345678 && sink) sink[0] = 1;
 }
 
+__global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, float* sink) {
+  // operands: fp16 values in (-1, 1) from a hash of the lane and the register
+  unsigned x = (unsigned)(blockIdx.x * 512 + threadIdx.x) * 2654435761u + 12345u;
+  auto next = [&]() {
+    x = x * 1664525u + 1013904223u;
+    return (half_t)((float)(int)(x >> 8) * (1.0f / 8388608.0f) - 1.0f);
+  };
+  h8 w[8], a[4];
+#pragma unroll
+  for (int o = 0; o < 8; o++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) w[o][e] = next();
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[i][e] = next();
+  f4 acc[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int o = 0; o < 8; o++) acc[i][o] = (f4){0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int o = 0; o < 8; o++)
+        acc[i][o] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[o], a[i], acc[i][o], 0, 0, 0);
+  }
+  f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int o = 0; o < 8; o++) sum += acc[i][o];
+  // sums of products of values below one stay far from this: nothing is written
+  if (sum[0] + sum[1] + sum[2] + sum[3] == 1.2345e30f && sink) sink[0] = 1.f;
+}
+
 int launch_probe_empty(int grid, hipStream_t stream) {
   hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(256), 0, stream);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  return launch_status();
 }
 
 int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream) {
   hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, a, (int*)nullptr);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  return launch_status();
+}
+
+int launch_probe_mfma(int grid, int iters, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3(grid), dim3(512), 0, stream, iters, (float*)nullptr);
+  return launch_status();
 }
 
 }  // namespace w4a16

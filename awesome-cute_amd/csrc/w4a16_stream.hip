@@ -622,7 +622,7 @@ static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
   constexpr int lds = StreamLds<MB, DEPTH, ONE_TILE>::kBytes;
   hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE>), dim3(grid), dim3(256), lds,
                      stream, a);
-  return hipGetLastError() == hipSuccess ? 0 : 3;
+  return launch_status();
 }
 
 template <int MB, bool GROUP, bool ONE_TILE>

@@ -306,7 +306,8 @@ def gemm_raw(entry, A, B, C, s, workspace, groupsize, thread_k=-1, thread_n=-1, 
 
 def probe(kind, B, n, k):
     """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
-    packed weights B with the streaming kernel's work split (marlin_amd_probe)."""
+    packed weights B with the streaming kernel's work split, 2 = a loop of nothing but MFMAs
+    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe)."""
     dev = B.get_device()
     rc = _lib.marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev))
     if rc != 0:

@@ -61,17 +61,35 @@ M_SWEEP = ["m32", "m64", "m128", "m256", "m512", "m1024"]
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE (KiB per dispatch) and scaled by what the same counters read for a
 # 256 MiB device copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 on this pool); the
-# summaries, with the commands, are under profiles/.
+# summaries, with the commands, are under profiles/.  Each entry names the plan
+# it was measured on (kernel, grid): when the library plans the shape otherwise
+# the figure is stale and is reported as null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode": int((4760.5 * 2.0 + 273.0) * 1024),         # 10.0 MB, 1.16 x algorithmic
-    "batch16": int((5688.5 * 2.0 + 2185.0) * 1024),       # 13.9 MB, 1.56 x (2 MiB of partial sums)
-    "prefill": int((33371.5 * 2.0 + 16393.0) * 1024),     # 85.1 MB, 2.02 x (A and B read by 16 tiles each)
-    "mlp_up": int((12296.0 * 2.0 + 1728.1) * 1024),       # 27.0 MB, 1.14 x
-    "mlp_down": int((13714.5 * 2.0 + 2185.0) * 1024),     # 30.3 MB, 1.28 x
-    "large_g128": int((66886.0 * 2.0 + 17930.5) * 1024),  # 155.3 MB, 1.23 x
-    "large_chan": int((65121.5 * 2.0 + 17930.5) * 1024),  # 151.7 MB, 1.24 x
-    "decode_large": int((59281.0 * 2.0 + 56.0) * 1024),   # 121.5 MB, 1.00 x
+    "decode": (("stream", 256), int((4760.5 * 2.0 + 273.0) * 1024)),          # 10.0 MB, 1.16 x algorithmic
+    "batch16": (("stream", 256), int((5688.5 * 2.0 + 2185.0) * 1024)),        # 13.9 MB, 1.56 x (2 MiB of partial sums)
+    "prefill": (("prefill", 256), int((33371.5 * 2.0 + 16393.0) * 1024)),     # 85.1 MB, 2.02 x (A and B read by 16 tiles each)
+    "mlp_up": (("stream", 172), int((12296.0 * 2.0 + 1728.1) * 1024)),        # 27.0 MB, 1.14 x
+    "mlp_down": (("stream", 256), int((13714.5 * 2.0 + 2185.0) * 1024)),      # 30.3 MB, 1.28 x
+    "large_g128": (("prefill", 224), int((66886.0 * 2.0 + 17930.5) * 1024)),  # 155.3 MB, 1.23 x
+    "large_chan": (("prefill", 224), int((65121.5 * 2.0 + 17930.5) * 1024)),  # 151.7 MB, 1.24 x
+    "decode_large": (("stream", 224), int((59281.0 * 2.0 + 56.0) * 1024)),    # 121.5 MB, 1.00 x
 }
+
+
+def algorithmic_bytes(M, N, K, g):
+    """weights + scales + activations + result, the bytes one GEMM has to move"""
+    return K * N // 2 + 2 * (K // 128 if g != -1 else 1) * N + 2 * M * K + 2 * M * N
+
+
+def sig(x, n=4):
+    """floats rounded to n significant digits (the printed line stays short)"""
+    if isinstance(x, float):
+        return float(f"{x:.{n}g}")
+    if isinstance(x, dict):
+        return {k: sig(v, n) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [sig(v, n) for v in x]
+    return x
 
 
 def build_inputs(torch, O, M, N, K, groupsize, nbuf, seed=0):
@@ -180,7 +198,7 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=Fal
     resident_ms = (graph_ms(torch, side, lambda i: call(0), steps, 1)[0]
                    if bound == "hbm" and nbuf > 1 else None)
     floor = None
-    if with_floor:
+    if with_floor and bound == "hbm":
         # what the launch alone and the weight stream alone cost, measured the same way
         e_ms, _ = graph_ms(torch, side, lambda i: marlin.probe(0, dBs[0], N, K), steps, 1)
         r_ms, r_spread = graph_ms(torch, side, lambda i: marlin.probe(1, dBs[i % nbuf], N, K),
@@ -188,9 +206,22 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=Fal
         floor = {"empty_kernel_us": e_ms * 1e3, "read_kernel_us": r_ms * 1e3,
                  "read_kernel_spread_us": [x * 1e3 for x in r_spread[:2]],
                  "read_GBps": weight_bytes / (r_ms * 1e-3) / 1e9,
-                 "what": "same grid and work split as the GEMM launch; read kernel = the packed "
-                         "weights through the streaming kernel's 128-bit loads, no arithmetic, "
-                         "nothing written; same buffer rotation and graph timing"}
+                 "what": "same grid and work split as a one-row launch of this shape; read kernel = "
+                         "the packed weights through the streaming kernel's 128-bit loads, no "
+                         "arithmetic, nothing written; same buffer rotation and graph timing"}
+    elif with_floor:
+        # what the matrix pipes sustain on the same count of multiply-adds with
+        # nothing beside them (one workgroup of 8 waves per CU, N*K/8192 MFMAs
+        # of 16384 flop per wave: the work of 2048 rows, scaled to M)
+        cus = marlin.device_info(0)["compute_units"]
+        per_wave = (N * K // 8192) // 32 * 32
+        probe_flops = cus * 8 * per_wave * 16384.0
+        m_ms, m_spread = graph_ms(torch, side, lambda i: marlin.probe(2, dBs[0], N, K), steps, 1)
+        sustained = probe_flops / (m_ms * 1e-3) / 1e12
+        floor = {"mfma_only_us": m_ms * 1e3, "mfma_only_flop": probe_flops,
+                 "sustained_TFLOPs": sustained,
+                 "what": "a loop of nothing but v_mfma_f32_16x16x32_f16 on pseudo-random operands, "
+                         "8 waves per CU with 32 independent accumulators each, same graph timing"}
 
     flops = 2.0 * M * N * K
     res = {
@@ -204,16 +235,33 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=Fal
         "weight_buffers_rotated": nbuf,
         "cache_resident_us_per_launch": None if resident_ms is None else resident_ms * 1e3,
     }
+    rc, plan = marlin.plan(M, N, K, g, -1, -1, -1, marlin.device_info(0)["compute_units"])
+    kernel = {1: "stream", 2: "prefill"}.get(plan["kernel"])
+    res["plan"] = {"kernel": kernel, "grid": plan["grid"], "k_slices": plan["k_slices"],
+                   "tile_rows": plan["tile_rows"]}
+    measured_on, traffic = MEASURED_TRAFFIC_BYTES.get(name, (None, None))
+    if measured_on != (kernel, plan["grid"]):
+        traffic = None  # measured on another plan: stale
     if bound == "hbm":
         ach = res["weight_GBps"]
         res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                           "frac": ach / HBM_PEAK_GBPS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+                           "frac": ach / HBM_PEAK_GBPS, "traffic": traffic}
+        if floor:
+            # the floor: a plain read of the same weights, launch included
+            res["roofline"]["floor_us"] = floor["read_kernel_us"]
+            res["roofline"]["frac_of_floor"] = floor["read_kernel_us"] / (ms * 1e3)
     else:
         ach = res["tflops"]
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": MFMA_FP16_PEAK_TFLOPS,
                            "unit": "TFLOP/s", "frac": ach / MFMA_FP16_PEAK_TFLOPS,
-                           "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+                           "traffic": traffic}
+        if floor:
+            # the floor: the same multiply-adds with nothing beside them
+            scaled = floor["mfma_only_us"] * flops / floor["mfma_only_flop"]
+            res["roofline"]["floor_us"] = scaled
+            res["roofline"]["frac_of_floor"] = scaled / (ms * 1e3)
+            res["roofline"]["sustained_peak"] = floor["sustained_TFLOPs"]
+    res["roofline"]["algorithmic_bytes"] = algorithmic_bytes(M, N, K, g)
     return res
 
 
@@ -239,11 +287,26 @@ def cpu_baseline(O, name, budget_s=12.0):
         reps1 += 1
     per1 = (time.perf_counter() - t1) / reps1
     return {"value": (K * N // 2) / per / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} full GEMMs of {name} (M={M} N={N} K={K} group={g}), "
-                      f"{per * 1e3:.1f} ms each, dequantise + fp32 GEMM, OpenMP",
+            "sample": f"{reps} {name} GEMMs (whole), {per * 1e3:.1f} ms each",
             "tflops": 2.0 * M * N * K / per / 1e12,
             "one_core": {"value": (K * N // 2) / per1 / 1e9, "unit": "GB/s", "cores": 1,
                          "sample": f"{reps1} GEMMs, {per1 * 1e3:.1f} ms each"}}
+
+
+def compact_row(r):
+    """one configuration in the printed line: shape [M, N, K, group], time,
+    fraction of the published peak of its roofline (HBM unless "b" says mfma),
+    the floor (a plain read of the weights, or the same MFMAs alone) and the
+    time's share of it, workgroups, HBM traffic over algorithmic bytes"""
+    rf = r["roofline"]
+    row = {"n": r["name"], "shape": [r["M"], r["N"], r["K"], r["groupsize"]],
+           "us": r["us_per_launch"], "frac": rf["frac"], "floor_us": rf.get("floor_us"),
+           "of_floor": rf.get("frac_of_floor"), "grid": r["plan"]["grid"]}
+    if rf["bound"] != "hbm":
+        row["b"] = rf["bound"]
+    if rf.get("traffic"):
+        row["traffic_x"] = rf["traffic"] / rf["algorithmic_bytes"]
+    return row
 
 
 def main():
@@ -255,6 +318,8 @@ def main():
                     help="headline (decode, then the other benchmark shapes) or one of: " +
                          ", ".join(SHAPES))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the sibling dense fp16 GEMM (reported with the details)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -292,20 +357,29 @@ def main():
 
     prop = torch.cuda.get_device_properties(0)
     info = marlin.device_info(0)  # from the HIP runtime, through the C ABI
-    # cross-check of the published matrix peak: CUs x 4 SIMDs x 1024 fp16 flop per clock x clock
+    # cross-check of the published matrix peak: CUs x 4 SIMDs x 1024 fp16 flop per clock x clock.
+    # (The published 8000 GB/s is 8192 pins x 8 Gb/s; the memory clock the runtime reports is
+    # printed as it is, no rate is derived from it.)
     clock_hz = info["clock_khz"] * 1e3
     peaks = {"hbm_GBps": HBM_PEAK_GBPS, "mfma_fp16_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
              "device": prop.name, "compute_units": info["compute_units"],
              "clock_MHz": info["clock_khz"] / 1e3,
              "mfma_fp16_TFLOPs_from_clock": info["compute_units"] * 4 * 1024 * clock_hz / 1e12,
              "memory_clock_MHz": info["memory_clock_khz"] / 1e3,
-             "memory_bus_bits": info["bus_width_bits"],
-             # HBM3E transfers twice per memory clock
-             "hbm_GBps_from_clock": info["memory_clock_khz"] * 1e3 * 2 * info["bus_width_bits"] / 8 / 1e9}
+             "memory_bus_bits": info["bus_width_bits"]}
     head = time_shape(torch, marlin, O, main_name, args.steps, args.warmup, with_floor=True)
-    shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup) for n in others]
+    shapes = [time_shape(torch, marlin, O, n, steps_for(n), args.warmup, with_floor=True)
+              for n in others]
+    for r in [head] + shapes:
+        if "sustained_peak" in r["roofline"]:
+            peaks["mfma_fp16_TFLOPs_sustained"] = r["roofline"]["sustained_peak"]
 
     M, N, K, g, bound = SHAPES[main_name]
+    # The printed line: the contract's fields, the headline's roofline (with its
+    # floor), the CPU baseline, and one short row per configuration -- short
+    # enough to survive whole wherever only the end of the output is kept.  The
+    # long form (spreads, eager rates, floors' parts, row-count sweep) goes to
+    # stderr before it.
     out = {
         "metric": "w4a16_gemm_weight_hbm_GBps" if bound == "hbm" else "w4a16_gemm_tflops",
         "value": head["weight_GBps"] if bound == "hbm" else head["tflops"],
@@ -314,49 +388,54 @@ def main():
         "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"{main_name}: M={M} N={N} K={K} groupsize={g} W4A16 GEMM",
-                   "weight_buffers_rotated": head["weight_buffers_rotated"],
-                   "timing": "K launches in one HIP graph, replayed for >= 50 ms and >= 20 "
-                             "replays, HIP events around every >= 200 launches, median sample"},
-        "us_per_launch_min_max": head["us_per_launch_min_max"],
-        "graph_replays": head["graph_replays"],
-        "stream_floor": head["stream_floor"],
-        "tflops": head["tflops"], "weight_GBps": head["weight_GBps"],
-        "cache_resident_us_per_launch": head["cache_resident_us_per_launch"],
-        "peaks": peaks,
-        "eager_ms_per_step": head["eager_ms_per_step"],
+        "config": {"workload": f"{main_name}: M={M} N={N} K={K} groupsize={g} W4A16 GEMM"},
         "roofline": head["roofline"],
-        "shapes": shapes,
-        "reference_published": {"RTX4090_marlin_cute_us": 8.714, "shape": "M=1 N=4096 K=4096 g=128",
-                                "note": "cache-warm kernel time on other hardware, not comparable"}
-        if main_name == "decode" else None,
     }
+    details = {"headline": head, "shapes": shapes, "peaks": peaks,
+               "timing": "K launches in one HIP graph, replayed for >= 50 ms and >= 20 replays, "
+                         "HIP events around every >= 200 launches, median sample",
+               "reference_published": {"RTX4090_marlin_cute_us": 8.714,
+                                       "shape": "M=1 N=4096 K=4096 g=128",
+                                       "note": "cache-warm kernel time on other hardware, "
+                                               "not comparable"}}
     if args.shape == "headline":
         sweep = []
         for n in M_SWEEP:
             r = time_shape(torch, marlin, O, n, min(args.steps, 400), args.warmup)
-            rc, plan = marlin.plan(r["M"], r["N"], r["K"], r["groupsize"], -1, -1, -1,
-                                   info["compute_units"])
             sweep.append({"M": r["M"], "N": r["N"], "K": r["K"], "groupsize": r["groupsize"],
                           "us_per_launch": r["us_per_launch"], "weight_GBps": r["weight_GBps"],
-                          "tflops": r["tflops"],
-                          "kernel": {1: "stream", 2: "prefill"}.get(plan["kernel"]),
-                          "grid": plan["grid"], "k_slices": plan["k_slices"],
-                          "tile_rows": plan["tile_rows"]})
-        out["m_sweep"] = sweep
+                          "tflops": r["tflops"], **r["plan"]})
+        details["m_sweep"] = sweep
+        # (decode_large is not one of the benchmark's configurations: details only)
+        out["rows"] = [compact_row(r) for r in [head] + shapes if r["name"] != "decode_large"]
+        out["m_sweep_us"] = {str(r["M"]): r["us_per_launch"] for r in sweep}
+        out["peaks"] = {"hbm_GBps": HBM_PEAK_GBPS, "mfma_TFLOPs": MFMA_FP16_PEAK_TFLOPS,
+                        "mfma_sustained_TFLOPs": peaks.get("mfma_fp16_TFLOPs_sustained")}
+    if args.extras:
         # the sibling dense fp16 GEMM with its stream-K tail, on the reference's three
         # examples (gemm/readme.md:29-31) and one problem small enough for 128 x 128
         # tiles; its own program is gemm_streamk.py
         import gemm_streamk
-        out["dense_streamk"] = [
+        details["dense_streamk"] = [
             {k: v for k, v in gemm_streamk.run(m, n, k, repeat=50, log=lambda *_: None).items()
              if k in ("value", "unit", "ms_per_step", "config", "roofline", "vendor_library_tflops",
                       "cos_similarity", "check")}
             for (m, n, k) in [(4096, 4352, 4096), (4096, 4352, 10240), (1152, 4352, 4096),
                               (2048, 2048, 2048)]]
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(O, main_name)
-    print(json.dumps(out))
+        cpu = cpu_baseline(O, main_name)
+        details["cpu_baseline"] = cpu
+        out["cpu_baseline"] = {k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample")}
+    print(json.dumps(sig(details)), file=sys.stderr)
+    # a table of the rows last on stderr, for whoever reads only its end
+    for r in [head] + shapes:
+        rf = r["roofline"]
+        print(f"{r['name']:12s} M={r['M']:<5d} N={r['N']:<6d} K={r['K']:<6d} g={r['groupsize']:<4d}"
+              f"{r['us_per_launch']:8.2f} us  {rf['frac']:.3f} of {rf['bound']} peak"
+              + (f"  floor {rf['floor_us']:.2f} us ({rf['frac_of_floor']:.2f})"
+                 if rf.get("floor_us") else ""), file=sys.stderr)
+    sys.stderr.flush()
+    print(json.dumps(sig(out)))
 
 
 if __name__ == "__main__":

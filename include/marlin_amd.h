@@ -81,9 +81,11 @@ int marlin_official(const void *A, const void *B, void *C, void *s, int prob_m, 
  * `sms` above the device's compute units with more than 16 rows can) returns
  * MARLIN_ERR_RUNTIME with a message.  All calls on one GPU share the array:
  * calls that may overlap in time on one GPU (different streams, or graph
- * branches) race on it and must use marlin_gemm instead.  The first call on a
- * device looks the array's address up and clears its counters with a kernel
- * on `stream`.
+ * branches) race on it -- silently: wrong sums, or a tile that nobody writes --
+ * and must use marlin_gemm instead.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress; no kernel, no allocation); the
+ * array's counters are zero when the library is loaded and every call hands
+ * them back zeroed.
  */
 int marlin_gemm_static(const void *A, const void *B, void *C, const void *s, int prob_m,
                        int prob_n, int prob_k, void *workspace, int groupsize, int dev,
@@ -182,12 +184,17 @@ long long marlin_amd_release(int dev);
 int marlin_amd_device_info(int dev, int *out);
 
 /*
- * Measurement probes on `stream` of the current device `dev`, with the grid
+ * Measurement probes on `stream` of device `dev`.  Kinds 0 and 1 use the grid
  * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
  * launch costs), kind 1 = a kernel that reads the packed weights B
  * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
  * 128-bit loads and does nothing with them (what the weight stream alone
- * costs).  Nothing is written.  No reference counterpart; for benchmarks.
+ * costs).  Kind 2 = a loop of nothing but v_mfma_f32_16x16x32_f16 on
+ * pseudo-random operands, one workgroup of 8 waves per compute unit and
+ * prob_n*prob_k/8192 MFMAs (16384 flop each) per wave, i.e. the multiply-adds
+ * of 2048 rows of this shape: what the matrix pipes sustain when nothing
+ * competes with them (B is not read).  Nothing is written.  No reference
+ * counterpart; for benchmarks.
  */
 int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
 
