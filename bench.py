@@ -67,7 +67,7 @@ M_SWEEP = ["m32", "m64", "m128", "m256", "m512", "m1024"]
 MEASURED_TRAFFIC_BYTES = {
     "decode": (("stream", 256), int((4760.5 * 2.0 + 273.0) * 1024)),          # 10.0 MB, 1.16 x algorithmic
     "batch16": (("stream", 256), int((5688.5 * 2.0 + 2185.0) * 1024)),        # 13.9 MB, 1.56 x (2 MiB of partial sums)
-    "prefill": (("prefill", 256), int((33371.5 * 2.0 + 16393.0) * 1024)),     # 85.1 MB, 2.02 x (A and B read by 16 tiles each)
+    "prefill": (("prefill", 256), int((33941.5 * 2.0 + 16389.5) * 1024)),     # 86.3 MB, 2.04 x (A and B read by 16 tiles each)
     "mlp_up": (("stream", 172), int((12296.0 * 2.0 + 1728.1) * 1024)),        # 27.0 MB, 1.14 x
     "mlp_down": (("stream", 256), int((13714.5 * 2.0 + 2185.0) * 1024)),      # 30.3 MB, 1.28 x
     "large_g128": (("prefill", 224), int((66886.0 * 2.0 + 17930.5) * 1024)),  # 155.3 MB, 1.23 x
