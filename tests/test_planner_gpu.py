@@ -1,0 +1,91 @@
+"""Guard of the host's kernel choice (marlin_host.hip: make_plan): on a dozen
+shapes between the decode and the prefill regime, the planned launch must not
+be more than 10 % slower than the best of the forced alternatives -- the
+streaming kernel, the prefill kernel on 64-row tiles and on 128-row tiles, each
+with the slice count its cost model picks.  The planner is a fitted cost model;
+this test is what fails when a kernel change shifts the costs under it.  (The
+dispatch rules it replaces: reference marlin_cute_kernel.cu:39-49.)
+"""
+import os
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
+
+SHAPES = [(m, n, k) for (n, k) in [(4096, 4096), (4096, 11008), (8192, 8192)]
+          for m in (48, 64, 128, 512)]
+SLACK = 1.10
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    import marlin
+    assert torch.cuda.is_available()
+    return torch, marlin
+
+
+def _us_per_call(torch, fn, reps):
+    """fastest of five timed runs of `reps` back-to-back calls"""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(5):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e3 / reps)
+    return best
+
+
+def _measure(torch, marlin, m, n, k):
+    dev = torch.device("cuda:0")
+    # enough distinct weight buffers that the stream comes from HBM, as in bench.py
+    nbuf = max(2, min(24, (600 << 20) // (k * n // 2)))
+    Bs = [torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev)
+          for _ in range(nbuf)]
+    S = (torch.rand((k // 128, n), device=dev) * 0.019 + 0.001).half()
+    A = torch.randn((m, k), device=dev).half()
+    C = torch.zeros((m, n), dtype=torch.half, device=dev)
+    ws = torch.zeros(n // 128 * 16, dtype=torch.int, device=dev)
+    turn = [0]
+
+    def call():
+        turn[0] += 1
+        marlin.mul(A, Bs[turn[0] % nbuf], C, S, ws)
+
+    times = {}
+    try:
+        times["planned"] = _us_per_call(torch, call, 40)
+        marlin.force_kernel(1)
+        times["streaming"] = _us_per_call(torch, call, 40)
+        for rows in (64, 128):
+            marlin.force_kernel(2)
+            marlin.force_tile_rows(rows)
+            times[f"prefill, {rows}-row tiles"] = _us_per_call(torch, call, 40)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_tile_rows(0)
+    torch.cuda.synchronize()
+    assert not ws.any().item()
+    return times
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_planned_launch_is_within_ten_percent_of_the_best_alternative(env, m, n, k):
+    torch, marlin = env
+    print(f"  planner guard m={m} n={n} k={k} plan={marlin.plan(m, n, k, 128)[1]}", flush=True)
+    for attempt in range(2):  # one re-measurement: timings of 15-60 us launches scatter by a few %
+        t = _measure(torch, marlin, m, n, k)
+        best = min(v for name, v in t.items() if name != "planned")
+        if t["planned"] <= SLACK * best:
+            return
+    raise AssertionError(f"m={m} n={n} k={k}: planned {t['planned']:.1f} us, alternatives {t}")
