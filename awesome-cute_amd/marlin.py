@@ -64,6 +64,15 @@ def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16, cut
     Asynchronous on the current stream of A's device.  Raises RuntimeError where
     the reference binding raises (marlin_gemm.cpp:27-31,48-55).
     """
+    if torch.compiler.is_compiling():
+        # under torch.compile the call is one opaque operator that mutates C and
+        # workspace (the reference advertises use within torch.compile, marlin.py:12)
+        return torch.ops.marlin_amd.mul(A, B, C, s, workspace, thread_k, thread_n, sms, max_par,
+                                        cute_version)
+    _mul_eager(A, B, C, s, workspace, thread_k, thread_n, sms, max_par, cute_version)
+
+
+def _mul_eager(A, B, C, s, workspace, thread_k, thread_n, sms, max_par, cute_version):
     if not (A.is_cuda and B.is_cuda and C.is_cuda and s.is_cuda and workspace.is_cuda):
         _complain((("A", A), ("B", B), ("C", C), ("s", s), ("workspace", workspace)), "is_cuda",
                   "must be a GPU tensor")
@@ -80,6 +89,22 @@ def mul(A, B, C, s, workspace, thread_k=-1, thread_n=-1, sms=-1, max_par=16, cut
                          err, 512)
     if rc != 0:
         raise RuntimeError(err.value.decode() or f"marlin_mul failed with code {rc}")
+
+
+# The same call as an operator of torch's dispatcher, for compilers that trace
+# Python: `mul` routes through it while torch.compile is tracing and calls the
+# library directly otherwise (the dispatcher costs more host time than the
+# one-row kernel takes).  It returns nothing; C and workspace are mutated.
+@torch.library.custom_op("marlin_amd::mul", mutates_args=("C", "workspace"))
+def _mul_op(A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, s: torch.Tensor,
+            workspace: torch.Tensor, thread_k: int, thread_n: int, sms: int, max_par: int,
+            cute_version: bool) -> None:
+    _mul_eager(A, B, C, s, workspace, thread_k, thread_n, sms, max_par, cute_version)
+
+
+@_mul_op.register_fake
+def _mul_fake(A, B, C, s, workspace, thread_k, thread_n, sms, max_par, cute_version):
+    return None
 
 
 def _complain(named, attr, what):

@@ -874,3 +874,68 @@ def test_graph_replays_match_eager(env, m, n, k):
             marlin.mul(d[3], d[4], C2, d[5], ws2)
             side.synchronize()
             assert torch.equal(C2, other)
+
+
+def test_mul_under_torch_compile(env):
+    """`marlin.mul` inside a function compiled with torch.compile(fullgraph=True)
+    (the reference advertises use within torch.compile, marlin.py:12): the call
+    is traced as the registered operator marlin_amd::mul, which mutates C and
+    the workspace, and the compiled function gives the oracle's result and the
+    eager call's bits, for a decode-sized and a prefill-sized problem."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+
+    def linear(A, B, s, ws):
+        C = torch.empty((A.shape[0], s.shape[1]), dtype=torch.half, device=A.device)
+        marlin.mul(A, B, C, s, ws)
+        return C * 2
+
+    compiled = torch.compile(linear, fullgraph=True, backend="aot_eager")
+    for (M, N, K, g) in [(4, 512, 1024, 128), (200, 768, 512, -1)]:
+        A, q, s, B, sp = O.make_problem(M, N, K, g, seed=M)
+        dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+        ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+        print(f"  torch.compile M={M} N={N} K={K} g={g}", flush=True)
+        got = compiled(dA, dB, ds, ws)
+        want = linear(dA, dB, ds, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and not ws.any().item()
+        r = O.compare((got / 2).cpu().numpy(), O.gemm(A, B, sp, N, g))
+        assert r.max_abs_err <= TOL * r.max_abs_ref
+    layer = marlin.Layer(512, 256, groupsize=128).to(dev)
+    A, q, s, B, sp = O.make_problem(8, 256, 512, 128, seed=5)
+    layer.B.copy_(torch.from_numpy(B))
+    layer.s.copy_(torch.from_numpy(sp))
+    got = torch.compile(layer, fullgraph=True, backend="aot_eager")(torch.from_numpy(A).to(dev))
+    torch.cuda.synchronize()
+    r = O.compare(got.cpu().numpy(), O.gemm(A, B, sp, 256, 128))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+
+
+@pytest.mark.parametrize("k", [8192, 21760])
+@pytest.mark.parametrize("kind", ["mean one", "all positive"])
+def test_per_channel_64_row_tiles_with_activations_of_one_sign(env, k, kind):
+    """Per-channel scales on 64-row prefill tiles accumulate biased integers
+    (1024 + n, 64 + n) and remove the bias, 1032 or 72 times the sum of the
+    activations, at the end: with activations of one sign that sum grows with
+    k, and so does the fp32 rounding it carries.  The result must stay inside
+    the mean-error bound (and far inside the max-error bound) all the same."""
+    torch, marlin = env
+    M, N = 64, 512
+    A, q, s, B, sp = O.make_problem(M, N, k, -1, seed=k)
+    rng = np.random.default_rng(k)
+    if kind == "mean one":
+        A = (1.0 + 0.25 * rng.standard_normal((M, k))).astype(np.float16)
+    else:
+        A = np.abs(rng.standard_normal((M, k))).astype(np.float16)
+    _force(marlin, kernel=2, rows=64)
+    try:
+        assert marlin.plan(M, N, k, -1)[1]["tile_rows"] == 64
+        C = gpu_gemm(env, A, B, sp, N)
+    finally:
+        _force(marlin)
+    r = O.compare(C, O.gemm(A, B, sp, N, -1))
+    print(f"  k={k} {kind}: max_abs_err {r.max_abs_err:.3e} of {r.max_abs_ref:.3e}, "
+          f"rel mean {r.rel_mean_abs_err:.2e}", flush=True)
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+    assert r.rel_mean_abs_err <= REL_MEAN_TOL

@@ -425,3 +425,47 @@ def test_marlin_lib_module_signature(marlin):
                                     "max_par", "cute_version"]
     d = {k: v.default for k, v in sig.parameters.items() if v.default is not inspect.Parameter.empty}
     assert d == {"thread_k": -1, "thread_n": -1, "sms": -1, "max_par": 8, "cute_version": True}
+
+
+def test_header_compiles_as_c_and_links(tmp_path):
+    """A consumer written in C: include/marlin_amd.h compiled with gcc -std=c11
+    -Wall -Werror (and as C++ with g++), linked against libmarlin_amd.so, the way
+    the reference's binding would be relinked (marlin_gemm.cpp:6-14, 34-46).
+    It asks marlin_amd_check for the reference's error codes and calls
+    marlin_gemm on an empty problem, which returns before touching a GPU."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "consumer.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include "marlin_amd.h"
+int main(void) {
+  /* k = 64 with thread_k = 128: the problem does not fit the tile */
+  if (marlin_amd_check(16, 256, 64, -1, 128, 128) != MARLIN_ERR_PROB_SHAPE) return 1;
+  /* group size 32: no kernel */
+  if (marlin_amd_check(16, 256, 512, 32, -1, -1) != MARLIN_ERR_KERN_SHAPE) return 2;
+  if (marlin_amd_check(16, 256, 512, 128, -1, -1) != MARLIN_OK) return 3;
+  /* an empty problem is fine and launches nothing (reference marlin_cute_kernel.cu:56-60) */
+  if (marlin_gemm(0, 0, 0, 0, 0, 256, 512, 0, 128, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 4;
+  if (marlin_cute(0, 0, 0, 0, 16, 0, 512, 0, -1, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 5;
+  if (marlin_official(0, 0, 0, 0, 16, 256, 0, 0, -1, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 6;
+  if (marlin_gemm_static(0, 0, 0, 0, 0, 256, 512, 0, 128, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 7;
+  printf("%s\n", marlin_amd_version());
+  return 0;
+}
+''')
+    libdir = os.path.join(ROOT, "awesome-cute_amd")
+    inc = os.path.join(ROOT, "include")
+    for cc, std in (("gcc", "-std=c11"), ("g++", "-std=c++11")):
+        exe = tmp_path / f"consumer_{cc}"
+        cmd = [cc, std, "-Wall", "-Werror", "-pedantic", "-I", inc]
+        cmd += ["-x", "c++"] if cc == "g++" else []
+        cmd += [str(src), "-o", str(exe), "-L", libdir, "-lmarlin_amd",
+                "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr
+        run = subprocess.run([str(exe)], capture_output=True, text=True)
+        assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+        assert "marlin_amd" in run.stdout

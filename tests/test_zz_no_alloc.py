@@ -133,3 +133,82 @@ def test_static_entry_in_a_graph(env):
         dA16 = torch.randn((16, K), dtype=torch.half, device=dev)
         assert marlin.gemm_raw("marlin_gemm_static", dA16, dB, other, ds, ws, g) == 0
         torch.cuda.synchronize()
+
+
+def test_static_entry_alone_allocates_nothing(env):
+    """Only marlin_gemm_static is called, after the pool has been emptied, on a
+    fresh stream: a shape whose column tiles are shared by 8 workgroups, then a
+    smaller one.  The pool stays empty and the device's free memory does not
+    move; the results are the oracle's."""
+    torch, marlin = env
+    dev = torch.device("cuda:0")
+    probs = []
+    for (M, N, K, g, seed) in [(16, 4096, 4096, 128, 21), (5, 1024, 2048, -1, 22)]:
+        A, q, s, B, sp = O.make_problem(M, N, K, g, seed)
+        dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+        dC = torch.full((M, N), 3.0, dtype=torch.half, device=dev)
+        ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+        probs.append(((A, B, sp, N, g), dA, dB, ds, dC, ws))
+    fresh = torch.cuda.Stream()
+    with torch.cuda.stream(fresh):
+        # the runtime sets a stream's queue up at its first launch (4 MiB of
+        # device memory on this pool): let a kernel of torch's pay for that
+        probs[0][5].add_(0)
+    torch.cuda.synchronize()
+    marlin.release()
+    assert marlin.scratch_bytes() == (0, 0)
+    free_before = torch.cuda.mem_get_info()[0]
+    for ((_, _, _, _, g), dA, dB, ds, dC, ws) in probs:
+        print(f"  marlin_gemm_static alone M={dA.shape[0]} N={dC.shape[1]} K={dA.shape[1]}", flush=True)
+        rc = marlin.gemm_raw("marlin_gemm_static", dA, dB, dC, ds, ws, g, stream=fresh.cuda_stream)
+        assert rc == 0, marlin.last_error()
+    fresh.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert marlin.scratch_bytes() == (0, 0)
+    for ((A, B, sp, N, g), dA, dB, ds, dC, ws) in probs:
+        assert not ws.any().item()
+        r = O.compare(dC.cpu().numpy(), O.gemm(A, B, sp, N, g))
+        assert r.max_abs_err <= TOL * r.max_abs_ref
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import sys
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[2])
+import numpy as np, torch, marlin, _oracle as O
+dev = torch.device("cuda:0")
+M, N, K, g = 4, 4096, 4096, 128
+A, q, s, B, sp = O.make_problem(M, N, K, g, 12)
+dA, dB, ds = (torch.from_numpy(x).to(dev) for x in (A, B, sp))
+dC = torch.zeros((M, N), dtype=torch.half, device=dev)
+ws = torch.zeros(N // 128 * 16, dtype=torch.int, device=dev)
+torch.cuda.synchronize()
+free_before = torch.cuda.mem_get_info()[0]
+side = torch.cuda.Stream()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph, stream=side):
+    # the first call of this process into the library
+    rc = marlin.gemm_raw("marlin_gemm_static", dA, dB, dC, ds, ws, g)
+assert rc == 0, marlin.last_error()
+assert marlin.scratch_bytes() == (0, 0)
+ref = O.gemm(A, B, sp, N, g)
+for _ in range(3):
+    dC.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    r = O.compare(dC.cpu().numpy(), ref)
+    assert r.max_abs_err <= 1e-2 * r.max_abs_ref and not ws.any().item()
+print("first call under capture: ok")
+"""
+
+
+def test_first_static_call_of_a_process_inside_a_capture(env):
+    """The very first call into the library is marlin_gemm_static under stream
+    capture (a process of its own, so that nothing has been set up before):
+    the device set-up and the symbol lookup must not break the capture, and
+    every replay gives the oracle's result."""
+    import subprocess
+    res = subprocess.run([sys.executable, "-c", _FIRST_CALL_UNDER_CAPTURE,
+                          os.path.join(ROOT, "awesome-cute_amd"), os.path.join(ROOT, "tests")],
+                         capture_output=True, text=True, timeout=300)
+    print(res.stdout[-2000:], res.stderr[-2000:], flush=True)
+    assert res.returncode == 0 and "first call under capture: ok" in res.stdout
