@@ -78,8 +78,8 @@ class Emitter:
     Loads and LDS operations complete in order of issue, each kind on its own
     counter.  wait_vm(reg) / wait_lgkm(reg) emit a wait that lets exactly the
     operations issued after the one that last wrote `reg` stay in flight.  The
-    loop body is generated twice by the caller; only the second copy is kept,
-    so that producers in the previous turn are counted right."""
+    caller emits the first turn of the loop as a copy of its own, so that the
+    loop's body finds a turn of the same order of issue before it."""
 
     def __init__(self):
         self.lines = []
@@ -342,10 +342,11 @@ def prologue(e, group):
         for op in range(13 if group else 9):
             for r in (0, 1):
                 unpack_op(e, group, 0, 0, (0, 1), j, op, r)
-    # everything requested so far has landed before the loop starts, so that
-    # the loop's waits, computed for its steady state, hold in its first turn
-    e.emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
-    e.drained(vm=True, lgkm=True)
+    # slab 0 is in LDS for everybody; the requests of stage 1 stay in flight
+    # (the first turn of the loop has waits of its own, computed from the order
+    # of issue above)
+    e.emit("s_waitcnt lgkmcnt(0)")
+    e.drained(lgkm=True)
     e.emit("s_barrier")
     for x in range(OPT["ahead"]):
         e.lds_read(AF(x), x * 256)
@@ -366,29 +367,38 @@ def epilogue(e):
     e.emit("s_waitcnt lgkmcnt(0)")
 
 
+def turn(e, group, label, back):
+    """two stages; leaves to .Lwd_done when the stages run out, else goes (or
+    falls through) to the steady loop"""
+    if label:
+        e.emit(f"{label}:")
+    stage(e, group, 0)
+    e.emit(f"s_add_i32 s{S_TMP}, s{S_CS}, 1")
+    e.emit(f"s_cmp_ge_i32 s{S_TMP}, s{S_STAGES}")
+    e.emit("s_cbranch_scc1 .Lwd_done_%=")
+    stage(e, group, 1)
+    e.emit(f"s_add_i32 s{S_CS}, s{S_CS}, 2")
+    if back:
+        e.emit(f"s_cmp_lt_i32 s{S_CS}, s{S_STAGES}")
+        e.emit("s_cbranch_scc1 .Lwd_loop_%=")
+    else:
+        e.emit(f"s_cmp_ge_i32 s{S_CS}, s{S_STAGES}")
+        e.emit("s_cbranch_scc1 .Lwd_done_%=")
+
+
 def generate(group):
     e = Emitter()
     prologue(e, group)
-    head = len(e.lines)
-    # the loop body twice: the first copy only sets up the issue history
-    for copy in (0, 1):
-        if copy == 1:
-            body_start = len(e.lines)
-        e.emit(".Lwd_loop_%=:")
-        stage(e, group, 0)
-        e.emit(f"s_add_i32 s{S_TMP}, s{S_CS}, 1")
-        e.emit(f"s_cmp_ge_i32 s{S_TMP}, s{S_STAGES}")
-        e.emit("s_cbranch_scc1 .Lwd_done_%=")
-        stage(e, group, 1)
-        e.emit(f"s_add_i32 s{S_CS}, s{S_CS}, 2")
-        e.emit(f"s_cmp_lt_i32 s{S_CS}, s{S_STAGES}")
-        e.emit("s_cbranch_scc1 .Lwd_loop_%=")
-    lines = e.lines[:head] + e.lines[body_start:]
-    e.lines = []
+    # The first turn is a copy of the loop's body with waits of its own: what is
+    # in flight when it starts was issued by the prologue, in another order
+    # than a turn of the loop leaves behind.  The loop's body follows; its
+    # waits see the first turn as the turn before, which issues exactly like
+    # the body itself.
+    turn(e, group, None, back=False)
+    turn(e, group, ".Lwd_loop_%=", back=True)
     e.emit(".Lwd_done_%=:")
     epilogue(e)
-    lines += e.lines
-    return lines
+    return e.lines
 
 
 def statement(group):
