@@ -1,8 +1,12 @@
-// Prefill W4A16 kernel (more than 64 activation rows): MFMA-bound, so the
-// design minimises everything that competes with the matrix pipe.
+// Prefill W4A16 kernel on 64-row tiles: 49 to 64 rows over big weights, and
+// more rows while twice as many tiles (against the 128-row tiles of
+// w4a16_prefill_wide.hip) save k slices.  With four row blocks every unpacked
+// weight word meets only four MFMAs, so the loop is bound by the unpack's issue
+// slots, not by the matrix pipe; the design keeps everything else out of their
+// way.
 //
 // One workgroup of 8 waves (two per SIMD) owns a 16*RB-row x 256-column tile
-// of C (RB = 8 row blocks, or 4: the host's choice) and, when the
+// of C (RB = 4 row blocks is the only instantiation) and, when the
 // tiles alone would leave compute units idle, one of `ksplit` slices of the k
 // range (the slices meet through the same ticketed exchange as the streaming
 // kernel's).  Waves 0-3 run the first half of the workgroup's k range and
@@ -24,8 +28,7 @@
 //     operand is one conflict-free ds_read_b128.
 // Per 32-deep k step a wave issues 4*RB MFMAs, RB + 2 LDS reads and the unpack
 // of 4 weight words (52 VALU instructions with group scales), software-
-// pipelined one step ahead and dealt out behind the MFMAs, two (RB = 8) or
-// four (RB = 4) per MFMA.
+// pipelined one step ahead and dealt out four behind every MFMA.
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
@@ -394,11 +397,8 @@ __global__ __launch_bounds__(512) void prefill_kernel(GemmArgs p, int tiles_m, i
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       const int cs = s + u;
-      // an odd count of stages: nothing is left for the second copy of the last
-      // turn (the count is the same for every wave of the workgroup).  Only
-      // with 128-row tiles: with 64 the exit costs the loop more than the
-      // stage of zeros that it saves.
-      if (RB == 8 && u == 1 && cs >= stages) break;
+      // (an odd count of stages computes one stage of zeros in the second copy
+      // of the last turn: an exit here costs this loop more than it saves)
       const int ring_next = ring == kPfRing - 1 ? 0 : ring + 1;
       const char* cur = smem + ring * kPfStageBytes;
       const char* nxt = smem + ring_next * kPfStageBytes;

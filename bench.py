@@ -4,15 +4,15 @@
 A step is one GEMM call (marlin.mul -> C ABI -> HIP kernel) on synthetic,
 seeded inputs already resident in HBM.  Memory-bound shapes rotate over enough
 distinct weight/scale buffers to exceed the 256 MB Infinity Cache, so the
-figure is an HBM figure and not a cache figure.  The K timed steps are captured
-in one HIP graph (kernel launches only) and bracketed by HIP events on the
-launch stream, so the host's launch cost is not part of the kernel's number.
-The graph is replayed until at least 50 ms of GPU time and 20 replays have been
-timed (each replay is exactly K steps; a pair of events brackets enough
-back-to-back replays to cover 200 launches; when K is smaller than the number
-of rotated weight buffers, several K-step graphs that continue the rotation
-take turns); `ms_per_step` is the median sample, the spread is reported
-beside it.  The eager (one host call per step) rate is
+figure is an HBM figure and not a cache figure.  The timed steps are captured in HIP
+graphs (kernel launches only) and bracketed by HIP events on the launch stream,
+so the host's launch cost is not part of the kernel's number: a graph holds a
+whole number of K-step runs, at least 200 launches (the hand-over between two
+graphs costs the GPU about 8 us, which is not the kernel's either), and is
+replayed until at least 50 ms of GPU time and 20 replays have been timed (when
+one graph does not cover the rotated weight buffers, several that continue the
+rotation take turns); `ms_per_step` is the median sample, the spread is
+reported beside it.  The eager (one host call per step) rate is
 reported next to it.
 
 Prints ONE JSON line: the headline workload is the decode configuration (
@@ -116,40 +116,42 @@ def build_inputs(torch, O, M, N, K, groupsize, nbuf, seed=0):
 
 
 def graph_ms(torch, side, fn, steps, period):
-    """Median time (ms) of one step over replays of graphs of exactly `steps`
-    calls fn(i).  i runs on from graph to graph, so `period` distinct buffers
-    are all visited even when steps < period.  Returns (median, (min, max,
-    samples))."""
-    n_graphs = max(1, min(8, -(-period // steps)))
+    """Median time (ms) of one step, calls fn(i), over replays of HIP graphs.
+
+    A graph holds a whole number of K-step runs, at least 200 launches: the
+    hand-over from one graph to the next costs the GPU about 8 us, which a
+    graph of 20 launches would spread over them as 0.4 us each (an empty
+    kernel: 1.94 us per launch in graphs of 20, 1.54 us in graphs of 200 or
+    2000), and that is the runtime's cost, not the kernel's.  i runs on from
+    graph to graph, so `period` distinct buffers are all visited.  Returns
+    (median, (min, max, samples))."""
+    per_graph = steps * max(1, -(-200 // steps))
+    n_graphs = max(1, min(8, -(-period // per_graph)))
     graphs = []
     for g in range(n_graphs):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
-            for i in range(steps):
-                fn(g * steps + i)
+            for i in range(per_graph):
+                fn(g * per_graph + i)
         graphs.append(graph)
     cur = torch.cuda.current_stream()
     for g in graphs:  # untimed: uploads the graph, brings the clocks up
         g.replay()
     torch.cuda.synchronize()
-    # one pair of events brackets `per_sample` back-to-back replays (at least
-    # 200 launches), so that what a graph launch costs by itself weighs little
-    per_sample = max(1, -(-200 // steps))
     times, total, r = [], 0.0, 0
     while (total < 50.0 or r < 20 or len(times) < 15) and r < 20000:
         batch = []
         for _ in range(5):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(cur)
-            for _ in range(per_sample):
-                graphs[r % n_graphs].replay()
-                r += 1
+            graphs[r % n_graphs].replay()
+            r += 1
             e1.record(cur)
             batch.append((e0, e1))
         torch.cuda.synchronize()
         for e0, e1 in batch:
             t = e0.elapsed_time(e1)
-            times.append(t / (steps * per_sample))
+            times.append(t / per_graph)
             total += t
     times.sort()
     return times[len(times) // 2], (times[0], times[-1], len(times))
@@ -392,8 +394,8 @@ def main():
         "roofline": head["roofline"],
     }
     details = {"headline": head, "shapes": shapes, "peaks": peaks,
-               "timing": "K launches in one HIP graph, replayed for >= 50 ms and >= 20 replays, "
-                         "HIP events around every >= 200 launches, median sample",
+               "timing": "HIP graphs of a whole number of K-step runs (>= 200 launches), replayed "
+                         "for >= 50 ms and >= 20 replays, HIP events around each replay, median",
                "reference_published": {"RTX4090_marlin_cute_us": 8.714,
                                        "shape": "M=1 N=4096 K=4096 g=128",
                                        "note": "cache-warm kernel time on other hardware, "
