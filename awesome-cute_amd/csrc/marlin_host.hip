@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "../../include/marlin_amd.h"
+#include "../../include/marlin_amd_tools.h"
 #include "scratch_pool.hpp"
 #include "w4a16_common.hpp"
 

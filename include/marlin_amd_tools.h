@@ -1,0 +1,95 @@
+/*
+ * Tools of libmarlin_amd.so beside its drop-in boundary (marlin_amd.h): what
+ * the library would do with a problem, per-thread overrides of its planner,
+ * and measurement probes.  None has a counterpart in the reference; tests and
+ * benchmarks use them, a binding of the W4A16 path does not need them.
+ */
+#ifndef MARLIN_AMD_TOOLS_H
+#define MARLIN_AMD_TOOLS_H
+
+#include "marlin_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Argument validation of marlin_gemm alone (no GPU touched): the code
+ * marlin_gemm would return for these sizes and hints. */
+int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                     int thread_n);
+
+/*
+ * How marlin_gemm would run a problem on a device with `cus` compute units:
+ * out[0] = kernel (0 = none, 1 = streaming, 2 = prefill), out[1] = workgroups,
+ * out[2] = granules per workgroup (streaming), out[3] = column tiles,
+ * out[4] = granules per column tile, out[5] = number of launches,
+ * out[6] = slices of the k range per tile (prefill), out[7] = rows of C per
+ * workgroup (prefill; 0 for the streaming kernel), out[8] = workgroups per
+ * column tile when the streaming kernel cuts every tile into that many runs
+ * (then out[2] is the longest run), 0 when it cuts the tile-major sequence of
+ * granules into equal runs of out[2]; out[9] = KiB of partial sums the launch
+ * exchanges through the library's scratch (0 = none).  `out` holds 10 ints.
+ * Returns the marlin_gemm error code for the shape.
+ */
+int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
+                    int thread_n, int sms, int cus, int *out);
+
+/*
+ * The streaming kernel's assignment of work to workgroups: out[b] is the work
+ * index of workgroup b of a launch of `grid` workgroups (work index w owns
+ * granules [w * granules_per_wg, (w + 1) * granules_per_wg) of the plan).  A
+ * permutation of 0..grid-1 in which the workgroups that the hardware deals to
+ * one XCD (b mod 8) hold consecutive indices.  No reference counterpart; for
+ * tests and tools.
+ */
+void marlin_amd_work_order(int grid, int *out);
+
+/*
+ * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
+ * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
+ * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is
+ * used).  Like the two overrides below it is kept per host thread, so it never
+ * changes what other threads' calls do.  No reference counterpart; for tests
+ * and tools.
+ */
+void marlin_amd_force_kernel(int which);
+
+/*
+ * Slices of the k range per tile of the prefill kernel, for the calling
+ * thread: 0 = choose by cost (default), n = n slices where the problem allows (each slice
+ * at least 256 deep).  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_k_slices(int slices);
+
+/*
+ * Rows of C per workgroup of the prefill kernel, for the calling thread: 0 =
+ * choose by cost (default), 64 or 128.  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_tile_rows(int rows);
+
+/*
+ * out[0..4] = compute units, shader clock (kHz), memory clock (kHz), memory
+ * bus width (bits), L2 size (bytes) of device dev, as the HIP runtime reports
+ * them.  Returns MARLIN_OK or MARLIN_ERR_RUNTIME.
+ */
+int marlin_amd_device_info(int dev, int *out);
+
+/*
+ * Measurement probes on `stream` of device `dev`.  Kinds 0 and 1 use the grid
+ * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
+ * launch costs), kind 1 = a kernel that reads the packed weights B
+ * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
+ * 128-bit loads and does nothing with them (what the weight stream alone
+ * costs).  Kind 2 = a loop of nothing but v_mfma_f32_16x16x32_f16 on
+ * pseudo-random operands, one workgroup of 8 waves per compute unit and
+ * prob_n*prob_k/8192 MFMAs (16384 flop each) per wave, i.e. the multiply-adds
+ * of 2048 rows of this shape: what the matrix pipes sustain when nothing
+ * competes with them (B is not read).  Nothing is written.  No reference
+ * counterpart; for benchmarks.
+ */
+int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
