@@ -83,7 +83,7 @@ def _measure(torch, marlin, m, n, k):
 def test_planned_launch_is_within_ten_percent_of_the_best_alternative(env, m, n, k):
     torch, marlin = env
     print(f"  planner guard m={m} n={n} k={k} plan={marlin.plan(m, n, k, 128)[1]}", flush=True)
-    for attempt in range(2):  # one re-measurement: timings of 15-60 us launches scatter by a few %
+    for attempt in range(3):  # re-measured twice at most: timings of 15-60 us launches scatter by a few %
         t = _measure(torch, marlin, m, n, k)
         best = min(v for name, v in t.items() if name != "planned")
         if t["planned"] <= SLACK * best:
