@@ -381,6 +381,40 @@ def test_prefill_kernel_tile_rows(env, rows, m, n, k, g):
         marlin.force_tile_rows(0)
 
 
+@pytest.mark.parametrize("m,n,k,g,slices", [
+    (128, 256, 64, -1, 0),      # one stage: the second k half has none
+    (129, 512, 192, -1, 0),     # three stages: halves of two and one
+    (256, 256, 320, -1, 0),     # five stages, leaves in the middle of the first turn
+    (100, 256, 384, 128, 0),
+    (128, 256, 512, 128, 2),    # two stages per half and slice
+    (1, 256, 256, 128, 0),      # one row of a 128-row tile
+    (127, 768, 640, 128, 0),    # a group's scales straddle the k halves
+    (128, 256, 1024, 128, 4),
+    (333, 1024, 4096, 128, 0),
+    (2048, 256, 8192, 128, 0),  # one column tile, many row tiles
+    (128, 256, 24576, 128, 0),  # a long k range per workgroup
+    (128, 256, 24576, 128, 8),
+])
+def test_four_wave_kernel_short_and_uneven_k_ranges(env, m, n, k, g, slices):
+    """The 128-row kernel's assembly loop at its ends: fewer stages than a turn
+    of the loop, odd counts (the k halves differ by a stage that reads zeros),
+    ranges that end inside the first turn, and long ones."""
+    torch, marlin = env
+    marlin.force_kernel(2)
+    marlin.force_tile_rows(128)
+    marlin.force_k_slices(slices)
+    try:
+        rc, plan = marlin.plan(m, n, k, g)
+        assert rc == 0 and plan["kernel"] == 2 and plan["tile_rows"] == 128
+        if slices:
+            assert plan["k_slices"] == slices
+        check(env, m, n, k, g, seed=m + k)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_tile_rows(0)
+        marlin.force_k_slices(0)
+
+
 @pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
 def test_frozen_known_answers(env, tag, groupsize):
     """The committed known answers (tests/golden): dequantised weights bit for
