@@ -1,4 +1,5 @@
-"""Builds libmarlin_amd.so (HIP kernels + C ABI) in-tree for gfx950."""
+"""Builds libmarlin_amd.so (HIP kernels + C ABI) and libmarlin_amd_probe.so (the
+measurement probes of the benchmark) in-tree for gfx950."""
 import os
 import subprocess
 import sys
@@ -6,6 +7,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmarlin_amd.so")
+PROBE_LIB = os.path.join(HERE, "libmarlin_amd_probe.so")
 # source -> extra flags.  The prefill kernel keeps its 128 accumulator registers
 # in ordinary VGPRs (it fits in 256), which spares the AGPR copy traffic the
 # default register split produces around every MFMA.
@@ -13,7 +15,6 @@ SOURCES = {
     "marlin_host.hip": [],
     "scratch_pool.hip": [],
     "w4a16_stream.hip": [],
-    "w4a16_probe.hip": [],
     "w4a16_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "w4a16_prefill_wide.hip": [],
     "f16_streamk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
@@ -51,6 +52,11 @@ def build_library(verbose=False):
         _run([HIPCC] + FLAGS + extra + ["-c", "-o", obj, os.path.join(CSRC, src)], verbose)
         objs.append(obj)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, verbose)
+    # the probes: a library of their own that asks the first one for its plans
+    obj = os.path.join(objdir, "w4a16_probe.o")
+    _run([HIPCC] + FLAGS + ["-c", "-o", obj, os.path.join(CSRC, "w4a16_probe.hip")], verbose)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB, obj, "-L", HERE,
+          "-lmarlin_amd", "-Wl,-rpath,$ORIGIN"], verbose)
     return LIB
 
 

@@ -593,48 +593,6 @@ int marlin_amd_device_info(int dev, int* out) {
   return MARLIN_OK;
 }
 
-int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, void* stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  int tk = -1, tn = -1;
-  int rc = check_shape(1, prob_n, prob_k, -1, tk, tn);
-  if (rc != MARLIN_OK) return rc;
-  if (prob_n == 0 || prob_k == 0 || dev < 0 || dev >= kMaxDevices || kind < 0 || kind > 2)
-    return MARLIN_ERR_PROB_SHAPE;
-  int prev = -1;
-  hipError_t e = hipGetDevice(&prev);
-  if (e == hipSuccess && prev != dev) e = hipSetDevice(dev);
-  if (e != hipSuccess) {
-    set_error(e, "hipSetDevice");
-    return MARLIN_ERR_RUNTIME;
-  }
-  const int cus = device_cus(dev);
-  rc = MARLIN_ERR_RUNTIME;
-  if (cus > 0) {
-    const PlanCtx cx = {cus, kPoolPartialLimit, Force()};
-    const Plan pl = make_plan(1, prob_n, prob_k, -1, cx);
-    (void)hipGetLastError();
-    if (kind == 0) {
-      rc = launch_probe_empty(pl.grid, stream);
-    } else if (kind == 1) {
-      GemmArgs a = {};
-      a.B = B;
-      a.M = 1;
-      a.N = prob_n;
-      a.K = prob_k;
-      a.gpb = pl.sp.gpb;
-      a.wpt = pl.sp.wpt;
-      rc = launch_probe_read(a, pl.grid, stream);
-    } else {
-      // one workgroup of 8 waves per CU; n*k/8192 MFMAs per wave (a multiple of 32)
-      const long long per_wave = (long long)prob_n * prob_k / 8192;
-      rc = launch_probe_mfma(cus, (int)(per_wave / 32 > 0 ? per_wave / 32 : 1), stream);
-    }
-    if (rc == MARLIN_ERR_RUNTIME) set_error(w4a16::last_launch_error(), "probe launch");
-  }
-  if (prev != dev) (void)hipSetDevice(prev);
-  return rc;
-}
-
 const char* marlin_amd_last_error(void) { return g_last_error; }
 
 const char* marlin_amd_version(void) { return "marlin_amd 0.2 (gfx950)"; }

@@ -201,13 +201,4 @@ int launch_prefill(const GemmArgs& a, bool group, int ksplit, hipStream_t stream
 int configure_prefill_wide_kernels();
 int launch_prefill_wide(const GemmArgs& a, bool group, int ksplit, hipStream_t stream);
 
-// Measurement probes (w4a16_probe.hip): an empty launch of `grid` workgroups,
-// and a plain read of the packed weights with the streaming kernel's work split
-// (a.B, a.N, a.K, a.gpb, a.wpt) and access pattern, no arithmetic.
-int launch_probe_empty(int grid, hipStream_t stream);
-int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream);
-// ... and a loop of nothing but MFMAs: grid workgroups of 8 waves, 32 * iters
-// v_mfma_f32_16x16x32_f16 per wave
-int launch_probe_mfma(int grid, int iters, hipStream_t stream);
-
 }  // namespace w4a16

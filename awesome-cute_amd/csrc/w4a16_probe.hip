@@ -1,5 +1,9 @@
-// Measurement probes: what a launch and a plain read of the packed weights cost
-// on this device, with no arithmetic, to judge the GEMM kernels against.
+// Measurement probes (libmarlin_amd_probe.so, include/marlin_amd_probe.h): what
+// a launch and a plain read of the packed weights cost on this device, with no
+// arithmetic, and what the matrix pipes sustain by themselves, to judge the
+// GEMM kernels against.  A library of its own, beside libmarlin_amd.so, which
+// it asks for the plan of the shape (marlin_amd_plan): the product library
+// carries no measurement code.
 //
 // probe_read_kernel walks the packed weights exactly as the streaming kernel
 // does for the same plan -- same work split, same workgroup-to-XCD order, same
@@ -9,6 +13,10 @@
 // a loop of nothing but v_mfma_f32_16x16x32_f16 on pseudo-random operands, two
 // waves per SIMD and 32 independent accumulators per wave: what the matrix
 // pipes of this board sustain when nothing competes with them.
+#include <cstdio>
+
+#include "../../include/marlin_amd_probe.h"
+#include "../../include/marlin_amd_tools.h"
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
@@ -105,19 +113,64 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, float* sink)
   if (sum[0] + sum[1] + sum[2] + sum[3] == 1.2345e30f && sink) sink[0] = 1.f;
 }
 
-int launch_probe_empty(int grid, hipStream_t stream) {
-  hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(256), 0, stream);
-  return launch_status();
-}
-
-int launch_probe_read(const GemmArgs& a, int grid, hipStream_t stream) {
-  hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, a, (int*)nullptr);
-  return launch_status();
-}
-
-int launch_probe_mfma(int grid, int iters, hipStream_t stream) {
-  hipLaunchKernelGGL(probe_mfma_kernel, dim3(grid), dim3(512), 0, stream, iters, (float*)nullptr);
-  return launch_status();
-}
-
 }  // namespace w4a16
+
+namespace {
+thread_local char g_probe_error[256] = "";
+}
+
+extern "C" {
+
+int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, void* stream_) {
+  using namespace w4a16;
+  hipStream_t stream = (hipStream_t)stream_;
+  g_probe_error[0] = 0;
+  if (prob_n <= 0 || prob_k <= 0 || dev < 0 || kind < 0 || kind > 2) return MARLIN_ERR_PROB_SHAPE;
+  int info[5] = {0, 0, 0, 0, 0};
+  if (marlin_amd_device_info(dev, info) != MARLIN_OK || info[0] <= 0) {
+    snprintf(g_probe_error, sizeof(g_probe_error), "device %d: %s", dev, marlin_amd_last_error());
+    return MARLIN_ERR_RUNTIME;
+  }
+  const int cus = info[0];
+  // the grid and the work split of a one-row launch of this shape
+  int plan[10];
+  const int rc = marlin_amd_plan(1, prob_n, prob_k, -1, -1, -1, -1, cus, plan);
+  if (rc != MARLIN_OK) return rc;
+  int prev = -1;
+  hipError_t e = hipGetDevice(&prev);
+  if (e == hipSuccess && prev != dev) e = hipSetDevice(dev);
+  if (e != hipSuccess) {
+    snprintf(g_probe_error, sizeof(g_probe_error), "hipSetDevice: %s", hipGetErrorString(e));
+    return MARLIN_ERR_RUNTIME;
+  }
+  (void)hipGetLastError();
+  const int grid = plan[1];
+  if (kind == 0) {
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(256), 0, stream);
+  } else if (kind == 1) {
+    GemmArgs a = {};
+    a.B = B;
+    a.M = 1;
+    a.N = prob_n;
+    a.K = prob_k;
+    a.gpb = plan[2];
+    a.wpt = plan[8];
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, stream, a, (int*)nullptr);
+  } else {
+    // one workgroup of 8 waves per CU; n*k/8192 MFMAs per wave (a multiple of 32)
+    const long long per_wave = (long long)prob_n * prob_k / 8192;
+    hipLaunchKernelGGL(probe_mfma_kernel, dim3(cus), dim3(512), 0, stream,
+                       (int)(per_wave / 32 > 0 ? per_wave / 32 : 1), (float*)nullptr);
+  }
+  e = hipGetLastError();
+  if (prev != dev) (void)hipSetDevice(prev);
+  if (e != hipSuccess) {
+    snprintf(g_probe_error, sizeof(g_probe_error), "probe launch: %s", hipGetErrorString(e));
+    return MARLIN_ERR_RUNTIME;
+  }
+  return MARLIN_OK;
+}
+
+const char* marlin_amd_probe_last_error(void) { return g_probe_error; }
+
+}  // extern "C"

@@ -33,8 +33,6 @@ _lib.marlin_amd_scratch_bytes.restype = ctypes.c_longlong
 _lib.marlin_amd_scratch_bytes.argtypes = [_I, _P]
 _lib.marlin_amd_release.restype = ctypes.c_longlong
 _lib.marlin_amd_release.argtypes = [_I]
-_lib.marlin_amd_probe.restype = _I
-_lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _P]
 _lib.marlin_amd_device_info.restype = _I
 _lib.marlin_amd_device_info.argtypes = [_I, _P]
 _lib.marlin_amd_check.restype = _I
@@ -329,14 +327,29 @@ def gemm_raw(entry, A, B, C, s, workspace, groupsize, thread_k=-1, thread_n=-1, 
                                 thread_k, thread_n, sms, max_par)
 
 
+_probe_lib = None
+
+
 def probe(kind, B, n, k):
     """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
     packed weights B with the streaming kernel's work split, 2 = a loop of nothing but MFMAs
-    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe)."""
+    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe, in the probe library
+    beside this one, loaded on first use)."""
+    global _probe_lib
+    if _probe_lib is None:
+        path = os.path.join(_HERE, "libmarlin_amd_probe.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it (python awesome-cute_amd/build.py)")
+        lib = ctypes.CDLL(path)
+        lib.marlin_amd_probe.restype = _I
+        lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _P]
+        lib.marlin_amd_probe_last_error.restype = ctypes.c_char_p
+        _probe_lib = lib
     dev = B.get_device()
-    rc = _lib.marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev))
+    rc = _probe_lib.marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev))
     if rc != 0:
-        raise RuntimeError(f"marlin_amd_probe failed with code {rc}: {last_error()}")
+        raise RuntimeError(f"marlin_amd_probe failed with code {rc}: "
+                           f"{_probe_lib.marlin_amd_probe_last_error().decode()}")
 
 
 def last_error():

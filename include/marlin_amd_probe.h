@@ -1,0 +1,41 @@
+/*
+ * libmarlin_amd_probe.so: measurement probes beside libmarlin_amd.so (which it
+ * links against for the plan of a shape).  They launch kernels that compute
+ * nothing -- an empty one, a plain read of the packed weights, a loop of MFMAs
+ * -- so that a benchmark can put the floor of the same box beside every GEMM
+ * time.  No counterpart in the reference; the product library contains none of
+ * this.
+ */
+#ifndef MARLIN_AMD_PROBE_H
+#define MARLIN_AMD_PROBE_H
+
+#include "marlin_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * A probe launch on `stream` of device `dev`.  Kinds 0 and 1 use the grid
+ * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
+ * launch costs), kind 1 = a kernel that reads the packed weights B
+ * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
+ * 128-bit loads and does nothing with them (what the weight stream alone
+ * costs).  Kind 2 = a loop of nothing but v_mfma_f32_16x16x32_f16 on
+ * pseudo-random operands, one workgroup of 8 waves per compute unit and
+ * prob_n*prob_k/8192 MFMAs (16384 flop each) per wave, i.e. the multiply-adds
+ * of 2048 rows of this shape: what the matrix pipes sustain when nothing
+ * competes with them (B is not read).  Nothing is written.  Returns
+ * MARLIN_OK, the marlin_gemm error code of the shape, or MARLIN_ERR_RUNTIME
+ * (text in marlin_amd_probe_last_error).
+ */
+int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
+
+
+/* Text of the calling thread's last probe failure ("" if none). */
+const char *marlin_amd_probe_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,8 +1,9 @@
 /*
  * Tools of libmarlin_amd.so beside its drop-in boundary (marlin_amd.h): what
- * the library would do with a problem, per-thread overrides of its planner,
- * and measurement probes.  None has a counterpart in the reference; tests and
- * benchmarks use them, a binding of the W4A16 path does not need them.
+ * the library would do with a problem, and per-thread overrides of its
+ * planner.  None has a counterpart in the reference; tests and benchmarks use
+ * them, a binding of the W4A16 path does not need them.  (The measurement
+ * probes are a library of their own: marlin_amd_probe.h.)
  */
 #ifndef MARLIN_AMD_TOOLS_H
 #define MARLIN_AMD_TOOLS_H
@@ -73,21 +74,6 @@ void marlin_amd_force_tile_rows(int rows);
  * them.  Returns MARLIN_OK or MARLIN_ERR_RUNTIME.
  */
 int marlin_amd_device_info(int dev, int *out);
-
-/*
- * Measurement probes on `stream` of device `dev`.  Kinds 0 and 1 use the grid
- * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
- * launch costs), kind 1 = a kernel that reads the packed weights B
- * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
- * 128-bit loads and does nothing with them (what the weight stream alone
- * costs).  Kind 2 = a loop of nothing but v_mfma_f32_16x16x32_f16 on
- * pseudo-random operands, one workgroup of 8 waves per compute unit and
- * prob_n*prob_k/8192 MFMAs (16384 flop each) per wave, i.e. the multiply-adds
- * of 2048 rows of this shape: what the matrix pipes sustain when nothing
- * competes with them (B is not read).  Nothing is written.  No reference
- * counterpart; for benchmarks.
- */
-int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
 
 #ifdef __cplusplus
 }

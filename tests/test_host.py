@@ -30,6 +30,7 @@ def marlin():
 def test_library_exports_every_declared_symbol(marlin):
     header = open(os.path.join(ROOT, "include", "marlin_amd.h")).read()
     tools = open(os.path.join(ROOT, "include", "marlin_amd_tools.h")).read()
+    probe = open(os.path.join(ROOT, "include", "marlin_amd_probe.h")).read()
     # the drop-in boundary carries no planner knob and no probe
     boundary = re.findall(r"\b(marlin_\w+)\s*\(", re.sub(r"/\*.*?\*/", "", header, flags=re.S))
     assert set(boundary) == {"marlin_gemm", "marlin_cute", "marlin_official", "marlin_mul",
@@ -43,11 +44,18 @@ def test_library_exports_every_declared_symbol(marlin):
             "marlin_amd_force_k_slices", "marlin_amd_force_tile_rows",
             "marlin_amd_last_error", "marlin_gemm_static", "marlin_gemm_static_capacity",
             "marlin_amd_scratch_bytes", "marlin_amd_release", "marlin_amd_device_info",
-            "marlin_amd_probe",
             "marlin_amd_version"} <= set(names)
     lib = ctypes.CDLL(LIB)
     for n in set(names):
         assert hasattr(lib, n), n
+    # the probes are a library of their own; the product library has none
+    probe_names = set(re.findall(r"\b(marlin_\w+)\s*\(", re.sub(r"/\*.*?\*/", "", probe, flags=re.S)))
+    assert probe_names == {"marlin_amd_probe", "marlin_amd_probe_last_error"}
+    assert not any(hasattr(lib, n) for n in probe_names)
+    assert b"probe" not in open(LIB, "rb").read()
+    plib = ctypes.CDLL(os.path.join(ROOT, "awesome-cute_amd", "libmarlin_amd_probe.so"))
+    for n in probe_names:
+        assert hasattr(plib, n), n
     assert b"gfx950" in marlin._lib.marlin_amd_version()
 
 
@@ -435,8 +443,9 @@ def test_marlin_lib_module_signature(marlin):
 
 
 def test_header_compiles_as_c_and_links(tmp_path):
-    """A consumer written in C: include/marlin_amd.h compiled with gcc -std=c11
-    -Wall -Werror (and as C++ with g++), linked against libmarlin_amd.so, the way
+    """A consumer written in C: the headers under include/ compiled with gcc
+    -std=c11 -Wall -Werror (and as C++ with g++), linked against libmarlin_amd.so
+    (and the probe library beside it), the way
     the reference's binding would be relinked (marlin_gemm.cpp:6-14, 34-46).
     It asks marlin_amd_check for the reference's error codes and calls
     marlin_gemm on an empty problem, which returns before touching a GPU."""
@@ -448,6 +457,7 @@ def test_header_compiles_as_c_and_links(tmp_path):
     src.write_text(r'''
 #include <stdio.h>
 #include "marlin_amd_tools.h"
+#include "marlin_amd_probe.h"
 int main(void) {
   /* k = 64 with thread_k = 128: the problem does not fit the tile */
   if (marlin_amd_check(16, 256, 64, -1, 128, 128) != MARLIN_ERR_PROB_SHAPE) return 1;
@@ -459,6 +469,9 @@ int main(void) {
   if (marlin_cute(0, 0, 0, 0, 16, 0, 512, 0, -1, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 5;
   if (marlin_official(0, 0, 0, 0, 16, 256, 0, 0, -1, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 6;
   if (marlin_gemm_static(0, 0, 0, 0, 0, 256, 512, 0, 128, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 7;
+  /* the probe library beside it: an unknown kind is refused before any GPU call */
+  if (marlin_amd_probe(7, 0, 256, 512, 0, 0) != MARLIN_ERR_PROB_SHAPE) return 8;
+  if (marlin_amd_probe_last_error()[0] != 0) return 9;
   printf("%s\n", marlin_amd_version());
   return 0;
 }
@@ -469,7 +482,7 @@ int main(void) {
         exe = tmp_path / f"consumer_{cc}"
         cmd = [cc, std, "-Wall", "-Werror", "-pedantic", "-I", inc]
         cmd += ["-x", "c++"] if cc == "g++" else []
-        cmd += [str(src), "-o", str(exe), "-L", libdir, "-lmarlin_amd",
+        cmd += [str(src), "-o", str(exe), "-L", libdir, "-lmarlin_amd_probe", "-lmarlin_amd",
                 "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"]
         res = subprocess.run(cmd, capture_output=True, text=True)
         assert res.returncode == 0, res.stderr
