@@ -53,28 +53,29 @@ __device__ __forceinline__ f4 load_partial(__amdgpu_buffer_rsrc_t r, int voffset
 
 }  // namespace
 
-// With one row block the activations of a granule travel through registers
-// and are transposed into LDS just before use (2 KiB per wave, inside the
-// 32 KiB that the cross-wave reduction uses later; barriers separate the two).
-// With more row blocks that would cost 8 registers per row block and ring
-// slot, so the activations are loaded straight into an LDS ring instead
-// (buffer_load ... lds, 16 bytes per lane) and never occupy a register before
-// they are an MFMA operand.
+// The activations of a granule travel through registers and are transposed
+// into LDS just before use (2 KiB per wave and row block, inside the memory
+// that the cross-wave reduction uses later; barriers separate the two): 8
+// registers per row block and ring slot.  Only the form whose workgroups cross
+// tile boundaries has no registers left for that with several row blocks (it
+// keeps two tiles' bookkeeping alive): there the activations are loaded
+// straight into an LDS ring instead (buffer_load ... lds, 16 bytes per lane).
+// Those loads are slow to issue -- with four row blocks a wave needs 1.7 us to
+// request its first two granules, against 1.0 us through registers -- so the
+// one-tile form, which every planned launch uses, does without them (M = 48,
+// N = K = 4096: 11.5 -> 10.7 us; M = 64: 13.9 -> 13.2; 8192 x 8192: 20.1 -> 19.7).
 template <int MB, int DEPTH, bool ONE_TILE>
 struct StreamLds {
-  static constexpr bool kDmaA = MB >= 2;
+  static constexpr bool kDmaA = MB >= 2 && !ONE_TILE;
   static constexpr int kReduceBytes = 32768;
   static constexpr int kRingBytesPerWave = kDmaA ? DEPTH * MB * 2048 : 0;
   // A workgroup that stays inside one tile reduces only once, after its last
-  // granule, when the ring is dead: the reduction then reuses the ring's
-  // memory, which leaves room for a deeper ring.
-  static constexpr bool kAliased = ONE_TILE && kDmaA;
-  static constexpr int kRingBase = kAliased ? 0 : kReduceBytes;
-  // ... and all row blocks are reduced in one pass (kReduceBytes each)
+  // granule, when the staging memory is dead: all row blocks are then reduced
+  // in one pass, kReduceBytes each, which also covers the staging (8 KiB x MB)
+  static constexpr bool kOnePass = ONE_TILE && MB >= 2;
+  static constexpr int kRingBase = kReduceBytes;
   static constexpr int kBytes =
-      kAliased ? (4 * kRingBytesPerWave > MB * kReduceBytes ? 4 * kRingBytesPerWave
-                                                            : MB * kReduceBytes)
-               : kReduceBytes + 4 * kRingBytesPerWave;
+      kOnePass ? MB * kReduceBytes : kReduceBytes + 4 * kRingBytesPerWave;
 };
 
 // 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at
@@ -332,11 +333,8 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // ---- sum the four waves; wave w ends up owning the 16-column groups
     // (j = w, h = 0/1) of every row block
     f4 res[MB][2];
-    // where the reduction reuses the ring's memory, the (empty) ring loads still
-    // in flight must have landed before anybody writes there
-    if constexpr (Lds::kAliased) __builtin_amdgcn_s_waitcnt(kWaitVm0);
     lds_barrier();
-    if constexpr (Lds::kAliased) {
+    if constexpr (Lds::kOnePass) {
       // room for all row blocks at once: two barriers instead of two per block
 #pragma unroll
       for (int i = 0; i < MB; i++) {
