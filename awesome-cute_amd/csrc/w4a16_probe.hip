@@ -113,11 +113,129 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, float* sink)
   if (sum[0] + sum[1] + sum[2] + sum[3] == 1.2345e30f && sink) sink[0] = 1.f;
 }
 
+// What a lone wave per SIMD can issue beside its MFMAs: 32 independent
+// v_mfma_f32_16x16x32_f16 per turn, each followed by NV independent packed-fp16
+// VALU operations, NL 16-byte LDS reads and NG 16-byte global loads (per 8
+// MFMAs for the two memory kinds).  Thread 0 of every workgroup writes the
+// cycles one turn took, averaged over the run; one workgroup of four waves per
+// CU (the LDS request keeps a second one out).
+template <int NV, int NL, int NG>
+__global__ __launch_bounds__(256) void probe_issue_kernel(int iters, const i4* src, float* out) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  unsigned x = (unsigned)(blockIdx.x * 256 + threadIdx.x) * 2654435761u + 12345u;
+  auto next = [&]() {
+    x = x * 1664525u + 1013904223u;
+    return (half_t)((float)(int)(x >> 8) * (1.0f / 8388608.0f) - 1.0f);
+  };
+  h8 w[8], a[4];
+#pragma unroll
+  for (int o = 0; o < 8; o++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) w[o][e] = next();
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[i][e] = next();
+  f4 acc[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int o = 0; o < 8; o++) acc[i][o] = (f4){0.f, 0.f, 0.f, 0.f};
+  h2 v[8];
+#pragma unroll
+  for (int r = 0; r < 8; r++) v[r] = (h2){next(), next()};
+  const h2 mul = {(half_t)0.999f, (half_t)1.001f};
+  i4 sink = {0, 0, 0, 0};
+  const unsigned lds_at = (unsigned)(size_t)(lds + threadIdx.x * 16);
+  const i4* g = src + threadIdx.x;
+  __syncthreads();
+  const unsigned long long t0 = __builtin_readcyclecounter();
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      i4 got_l[NL > 0 ? NL : 1], got_g[NG > 0 ? NG : 1];
+#pragma unroll
+      for (int o = 0; o < 8; o++) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[i][o]) : "v"(w[o]), "v"(a[i]));
+#pragma unroll
+        for (int r = 0; r < NV; r++)
+          asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(v[(o * NV + r) & 7]) : "v"(mul));
+        if (o < NL) asm volatile("ds_read_b128 %0, %1" : "=v"(got_l[o]) : "v"(lds_at) : "memory");
+        if (o < NG)
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(got_g[o]) : "v"(g + 256 * o) : "memory");
+      }
+      // the loads of this row block are consumed before the next one's are issued
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int o = 0; o < NL; o++) sink |= got_l[o];
+#pragma unroll
+      for (int o = 0; o < NG; o++) sink |= got_g[o];
+    }
+  }
+  const unsigned long long t1 = __builtin_readcyclecounter();
+  f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int o = 0; o < 8; o++) sum += acc[i][o];
+  float keep = sum[0] + sum[1] + sum[2] + sum[3];
+#pragma unroll
+  for (int r = 0; r < 8; r++) keep += (float)v[r][0] + (float)v[r][1];
+  if (threadIdx.x == 0)
+    out[blockIdx.x] = (float)(t1 - t0) / (float)iters +
+                      ((keep == 1.2345e30f || sink[0] == 0x12345678) ? 1.f : 0.f);
+}
+
+// What one CU pulls from memory: every workgroup of 256 threads reads its own
+// `bytes_per_wg` of `src` with `depth` 16-byte loads in flight per thread and
+// writes the time it took in ticks of the 100 MHz constant clock (thread 0) --
+// with one workgroup the figure is one CU's, with one per CU the whole chip's.
+template <int DEPTH>
+__global__ __launch_bounds__(256) void probe_pull_kernel(const i4* src, int pieces_per_thread,
+                                                         float* out) {
+  const i4* g = src + (size_t)blockIdx.x * 256 * pieces_per_thread + threadIdx.x;
+  i4 acc = {0, 0, 0, 0};
+  __syncthreads();
+  const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+  for (int p = 0; p < pieces_per_thread; p += DEPTH) {
+    i4 got[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+      got[d] = __builtin_nontemporal_load(g + (size_t)(p + d) * 256);
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) acc |= got[d];
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0)
+    out[blockIdx.x] = (float)(t1 - t0) + ((acc[0] & acc[1]) == 0x12345678 ? 1.f : 0.f);
+}
+
 }  // namespace w4a16
 
 namespace {
 thread_local char g_probe_error[256] = "";
+
+bool probe_fail(const char* what, hipError_t e) {
+  snprintf(g_probe_error, sizeof(g_probe_error), "%s: %s", what, hipGetErrorString(e));
+  return false;
 }
+
+// launch `fn` (which enqueues one kernel writing n floats to dev_out), wait,
+// bring the floats to `host_out`
+template <class F>
+bool run_and_fetch(int n, float* host_out, F fn) {
+  float* dev_out = nullptr;
+  hipError_t e = hipMalloc((void**)&dev_out, (size_t)n * sizeof(float));
+  if (e != hipSuccess) return probe_fail("hipMalloc", e);
+  (void)hipGetLastError();
+  fn(dev_out);
+  e = hipGetLastError();
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpy(host_out, dev_out, (size_t)n * sizeof(float), hipMemcpyDeviceToHost);
+  (void)hipFree(dev_out);
+  return e == hipSuccess ? true : probe_fail("probe launch", e);
+}
+}  // namespace
 
 extern "C" {
 
@@ -169,6 +287,72 @@ int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, v
     return MARLIN_ERR_RUNTIME;
   }
   return MARLIN_OK;
+}
+
+int marlin_amd_probe_issue(int n_valu, int n_lds, int n_global, int iters, int workgroups,
+                           float* cycles_out) {
+  using namespace w4a16;
+  g_probe_error[0] = 0;
+  if (iters <= 0 || workgroups <= 0 || workgroups > 4096 || !cycles_out)
+    return MARLIN_ERR_PROB_SHAPE;
+  i4* src = nullptr;
+  hipError_t e = hipMalloc((void**)&src, 256 * 8 * sizeof(i4));
+  if (e != hipSuccess) {
+    probe_fail("hipMalloc", e);
+    return MARLIN_ERR_RUNTIME;
+  }
+  (void)hipMemset(src, 0, 256 * 8 * sizeof(i4));
+  const int lds = 96 * 1024;  // more than half a CU's: one workgroup per CU
+  bool ok = false, known = true;
+  auto go = [&](auto kernel) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds) !=
+        hipSuccess)
+      return probe_fail("hipFuncSetAttribute", hipGetLastError());
+    return run_and_fetch(workgroups, cycles_out, [&](float* out) {
+      hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(256), lds, 0, iters, (const i4*)src, out);
+    });
+  };
+  const int key = n_valu * 100 + n_lds * 10 + n_global;
+  switch (key) {
+    case 0: ok = go(probe_issue_kernel<0, 0, 0>); break;
+    case 100: ok = go(probe_issue_kernel<1, 0, 0>); break;
+    case 200: ok = go(probe_issue_kernel<2, 0, 0>); break;
+    case 300: ok = go(probe_issue_kernel<3, 0, 0>); break;
+    case 400: ok = go(probe_issue_kernel<4, 0, 0>); break;
+    case 10: ok = go(probe_issue_kernel<0, 1, 0>); break;
+    case 20: ok = go(probe_issue_kernel<0, 2, 0>); break;
+    case 1: ok = go(probe_issue_kernel<0, 0, 1>); break;
+    case 2: ok = go(probe_issue_kernel<0, 0, 2>); break;
+    case 210: ok = go(probe_issue_kernel<2, 1, 0>); break;
+    case 201: ok = go(probe_issue_kernel<2, 0, 1>); break;
+    default: known = false;
+  }
+  (void)hipFree(src);
+  if (!known) return MARLIN_ERR_PROB_SHAPE;
+  return ok ? MARLIN_OK : MARLIN_ERR_RUNTIME;
+}
+
+int marlin_amd_probe_pull(const void* src, long long src_bytes, long long bytes_per_workgroup,
+                          int depth, int workgroups, float* cycles_out) {
+  using namespace w4a16;
+  g_probe_error[0] = 0;
+  const long long pieces = bytes_per_workgroup / (256 * 16);
+  if (!src || !cycles_out || workgroups <= 0 || workgroups > 4096 || pieces <= 0 ||
+      pieces > (1 << 20) || pieces % 16 != 0 || pieces * 256 * 16 * workgroups > src_bytes)
+    return MARLIN_ERR_PROB_SHAPE;
+  bool ok;
+  auto go = [&](auto kernel) {
+    return run_and_fetch(workgroups, cycles_out, [&](float* out) {
+      hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(256), 0, 0, (const i4*)src, (int)pieces, out);
+    });
+  };
+  switch (depth) {
+    case 1: ok = go(probe_pull_kernel<1>); break;
+    case 4: ok = go(probe_pull_kernel<4>); break;
+    case 16: ok = go(probe_pull_kernel<16>); break;
+    default: return MARLIN_ERR_PROB_SHAPE;
+  }
+  return ok ? MARLIN_OK : MARLIN_ERR_RUNTIME;
 }
 
 const char* marlin_amd_probe_last_error(void) { return g_probe_error; }

@@ -330,11 +330,8 @@ def gemm_raw(entry, A, B, C, s, workspace, groupsize, thread_k=-1, thread_n=-1, 
 _probe_lib = None
 
 
-def probe(kind, B, n, k):
-    """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
-    packed weights B with the streaming kernel's work split, 2 = a loop of nothing but MFMAs
-    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe, in the probe library
-    beside this one, loaded on first use)."""
+def _probes():
+    """The probe library beside this one (libmarlin_amd_probe.so), loaded on first use."""
     global _probe_lib
     if _probe_lib is None:
         path = os.path.join(_HERE, "libmarlin_amd_probe.so")
@@ -343,13 +340,49 @@ def probe(kind, B, n, k):
         lib = ctypes.CDLL(path)
         lib.marlin_amd_probe.restype = _I
         lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _P]
+        lib.marlin_amd_probe_issue.restype = _I
+        lib.marlin_amd_probe_issue.argtypes = [_I, _I, _I, _I, _I, _P]
+        lib.marlin_amd_probe_pull.restype = _I
+        lib.marlin_amd_probe_pull.argtypes = [_P, ctypes.c_longlong, ctypes.c_longlong, _I, _I, _P]
         lib.marlin_amd_probe_last_error.restype = ctypes.c_char_p
         _probe_lib = lib
-    dev = B.get_device()
-    rc = _probe_lib.marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev))
+    return _probe_lib
+
+
+def _probe_check(rc, what):
     if rc != 0:
-        raise RuntimeError(f"marlin_amd_probe failed with code {rc}: "
-                           f"{_probe_lib.marlin_amd_probe_last_error().decode()}")
+        raise RuntimeError(f"{what} failed with code {rc}: "
+                           f"{_probes().marlin_amd_probe_last_error().decode()}")
+
+
+def probe(kind, B, n, k):
+    """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
+    packed weights B with the streaming kernel's work split, 2 = a loop of nothing but MFMAs
+    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe)."""
+    dev = B.get_device()
+    _probe_check(_probes().marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev)),
+                 "marlin_amd_probe")
+
+
+def probe_issue(n_valu, n_lds=0, n_global=0, iters=2000, workgroups=256):
+    """Shader cycles per MFMA of a lone wave per SIMD that issues, behind every MFMA, n_valu
+    packed-fp16 VALU operations and, behind the first n_lds / n_global of every eight, a 16-byte
+    LDS read / global load: median over the workgroups (marlin_amd_probe_issue)."""
+    out = (ctypes.c_float * workgroups)()
+    _probe_check(_probes().marlin_amd_probe_issue(n_valu, n_lds, n_global, iters, workgroups, out),
+                 "marlin_amd_probe_issue")
+    return float(np.median(np.frombuffer(out, dtype=np.float32))) / 32.0
+
+
+def probe_pull(src, bytes_per_workgroup, depth, workgroups):
+    """Microseconds every one of `workgroups` workgroups needs to read its own
+    bytes_per_workgroup of the tensor `src` with `depth` 16-byte loads in flight per thread
+    (marlin_amd_probe_pull; the kernel's own 100 MHz clock)."""
+    out = (ctypes.c_float * workgroups)()
+    _probe_check(_probes().marlin_amd_probe_pull(src.data_ptr(), src.numel() * src.element_size(),
+                                                 bytes_per_workgroup, depth, workgroups, out),
+                 "marlin_amd_probe_pull")
+    return np.frombuffer(out, dtype=np.float32) / 100.0
 
 
 def last_error():

@@ -311,6 +311,42 @@ def compact_row(r):
     return row
 
 
+def hardware_facts(torch, marlin):
+    """The figures of this board that shaped the kernels, each from a probe kernel of the
+    probe library (libmarlin_amd_probe.so); shader cycles are the wave's own counter."""
+    clock_ghz = marlin.device_info()["clock_khz"] / 1e6
+    print(f"device clock {clock_ghz:.2f} GHz (nominal); one workgroup of four waves per CU, "
+          "32 independent v_mfma_f32_16x16x32_f16 per turn")
+    print("cycles per MFMA of a lone wave per SIMD that also issues ...")
+    base = marlin.probe_issue(0)
+    rows = [("nothing else", (0, 0, 0)), ("1 packed-fp16 VALU per MFMA", (1, 0, 0)),
+            ("2 VALU per MFMA", (2, 0, 0)), ("3 VALU per MFMA", (3, 0, 0)),
+            ("4 VALU per MFMA", (4, 0, 0)), ("1 ds_read_b128 per 8 MFMAs", (0, 1, 0)),
+            ("2 ds_read_b128 per 8 MFMAs", (0, 2, 0)), ("1 global 16-byte load per 8 MFMAs", (0, 0, 1)),
+            ("2 global loads per 8 MFMAs", (0, 0, 2)),
+            ("2 VALU per MFMA and 1 ds_read_b128 per 8", (2, 1, 0)),
+            ("2 VALU per MFMA and 1 global load per 8", (2, 0, 1))]
+    for label, (nv, nl, ng) in rows:
+        c = marlin.probe_issue(nv, nl, ng)
+        extra = ""
+        if nl + ng and nv == 0:
+            extra = f"  ({(c - base) * 8 / (nl + ng):.1f} cycles per memory instruction)"
+        elif nv and not (nl + ng):
+            extra = f"  ({(c - base) / nv:.1f} cycles per VALU operation beyond the MFMA's own time)"
+        print(f"  {label:45s} {c:6.2f}{extra}")
+    print("what compute units pull from memory (16-byte loads per thread, 256 threads a workgroup; "
+          "slowest workgroup, by the kernel's 100 MHz clock):")
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    src.random_(0, 255)
+    cus = marlin.device_info()["compute_units"]
+    for wgs, per_wg in ((1, 16 << 20), (cus, 4 << 20)):
+        for depth in (1, 4, 16):
+            us = marlin.probe_pull(src, per_wg, depth, wgs)
+            gbps = per_wg * wgs / (float(us.max()) * 1e-6) / 1e9
+            print(f"  {wgs:4d} workgroup(s) x {per_wg >> 20} MiB, {depth:2d} loads in flight per thread: "
+                  f"{gbps / wgs:7.1f} GB/s per CU, {gbps:8.0f} GB/s together")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -325,6 +361,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--facts", action="store_true",
+                    help="instead of the benchmark: the hardware figures the design leans on, "
+                         "measured by the probe library (what one wave issues beside its MFMAs, "
+                         "what compute units pull from memory); a table on stdout")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus must be 1 "
@@ -335,6 +375,10 @@ def main():
     import _oracle as O
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    if args.facts:
+        hardware_facts(torch, marlin)
+        return
 
     if args.shape == "headline":
         main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128",

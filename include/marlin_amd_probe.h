@@ -31,6 +31,28 @@ extern "C" {
  */
 int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
 
+/*
+ * What a lone wave per SIMD can issue beside its MFMAs (synchronous, on the
+ * current device's null stream): `workgroups` workgroups of four waves, one per
+ * CU, run `iters` turns of 32 independent v_mfma_f32_16x16x32_f16, each MFMA
+ * followed by n_valu independent packed-fp16 VALU operations (0..4), and the
+ * first n_lds / n_global MFMAs of every eight also by a 16-byte LDS read / a
+ * 16-byte global load (supported mixes: n_valu alone; n_lds 1, 2 or n_global
+ * 1, 2 alone; n_valu = 2 with one of either).  cycles_out[w] = shader cycles
+ * per turn of workgroup w (divide by 32 for cycles per MFMA).
+ */
+int marlin_amd_probe_issue(int n_valu, int n_lds, int n_global, int iters, int workgroups,
+                           float *cycles_out);
+
+/*
+ * What compute units pull from memory (synchronous, null stream): workgroup w
+ * of 256 threads reads bytes_per_workgroup (a multiple of 64 KiB) of `src`
+ * (src_bytes long, at least workgroups * bytes_per_workgroup) starting at
+ * w * bytes_per_workgroup with `depth` (1, 4 or 16) 16-byte loads in flight per
+ * thread; ticks_out[w] = what it took in ticks of the 100 MHz constant clock.
+ */
+int marlin_amd_probe_pull(const void *src, long long src_bytes, long long bytes_per_workgroup,
+                          int depth, int workgroups, float *ticks_out);
 
 /* Text of the calling thread's last probe failure ("" if none). */
 const char *marlin_amd_probe_last_error(void);

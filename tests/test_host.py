@@ -50,7 +50,8 @@ def test_library_exports_every_declared_symbol(marlin):
         assert hasattr(lib, n), n
     # the probes are a library of their own; the product library has none
     probe_names = set(re.findall(r"\b(marlin_\w+)\s*\(", re.sub(r"/\*.*?\*/", "", probe, flags=re.S)))
-    assert probe_names == {"marlin_amd_probe", "marlin_amd_probe_last_error"}
+    assert probe_names == {"marlin_amd_probe", "marlin_amd_probe_issue", "marlin_amd_probe_pull",
+                           "marlin_amd_probe_last_error"}
     assert not any(hasattr(lib, n) for n in probe_names)
     assert b"probe" not in open(LIB, "rb").read()
     plib = ctypes.CDLL(os.path.join(ROOT, "awesome-cute_amd", "libmarlin_amd_probe.so"))
