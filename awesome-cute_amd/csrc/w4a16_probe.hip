@@ -150,28 +150,36 @@ __global__ __launch_bounds__(256) void probe_issue_kernel(int iters, const i4* s
   const i4* g = src + threadIdx.x;
   __syncthreads();
   const unsigned long long t0 = __builtin_readcyclecounter();
+  // the loads of a row block are consumed one row block later (eight MFMAs,
+  // more than their latency from LDS or a cache hit), so that what is measured
+  // is what issuing them costs, not the wait for them
+  i4 got_l[2][NL > 0 ? NL : 1] = {}, got_g[2][NG > 0 ? NG : 1] = {};
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      i4 got_l[NL > 0 ? NL : 1], got_g[NG > 0 ? NG : 1];
 #pragma unroll
       for (int o = 0; o < 8; o++) {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[i][o]) : "v"(w[o]), "v"(a[i]));
 #pragma unroll
         for (int r = 0; r < NV; r++)
           asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(v[(o * NV + r) & 7]) : "v"(mul));
-        if (o < NL) asm volatile("ds_read_b128 %0, %1" : "=v"(got_l[o]) : "v"(lds_at) : "memory");
+        if (o < NL)
+          asm volatile("ds_read_b128 %0, %1" : "=v"(got_l[i & 1][o]) : "v"(lds_at) : "memory");
         if (o < NG)
-          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(got_g[o]) : "v"(g + 256 * o) : "memory");
+          asm volatile("global_load_dwordx4 %0, %1, off"
+                       : "=v"(got_g[i & 1][o])
+                       : "v"(g + 256 * o)
+                       : "memory");
       }
-      // the loads of this row block are consumed before the next one's are issued
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      // all but this row block's loads have landed
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(%1)" ::"n"(NG), "n"(NL) : "memory");
 #pragma unroll
-      for (int o = 0; o < NL; o++) sink |= got_l[o];
+      for (int o = 0; o < NL; o++) sink |= got_l[(i & 1) ^ 1][o];
 #pragma unroll
-      for (int o = 0; o < NG; o++) sink |= got_g[o];
+      for (int o = 0; o < NG; o++) sink |= got_g[(i & 1) ^ 1][o];
     }
   }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   const unsigned long long t1 = __builtin_readcyclecounter();
   f4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
