@@ -124,6 +124,8 @@ struct Plan {
   int ksplit;            // prefill: slices of the k range per tile
   int tile_rows;         // prefill: rows of C per workgroup
   size_t partial_bytes;  // fp32 partial sums the launch exchanges through scratch (0: none)
+  int row_halves;        // streaming, one-tile form: 2 when the rows are cut into two halves
+  int half_rows;         // rows of the first half
 };
 
 constexpr int kStreamMaxRows = 64;
@@ -134,6 +136,7 @@ constexpr int kStreamMaxRows = 64;
 // rows of C per prefill workgroup (0 = by cost, 64 or 128).
 struct Force {
   int kernel = 0, k_slices = 0, tile_rows = 0;
+  int row_halves = 0;  // streaming kernel: 0 = by cost, 1 = never cut the rows, 2 = cut them where possible
 };
 thread_local Force t_force;
 
@@ -143,6 +146,7 @@ struct PlanCtx {
   int cus;
   size_t partial_limit;
   Force force;
+  bool two_counters = true;  // the workspace has room for two counters per column tile
 };
 
 // Cost in us of the prefill kernel with `tiles` tiles of tile_rows rows cut into
@@ -264,6 +268,30 @@ StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
   return sp;
 }
 
+// What cutting the rows of a streaming launch in two saves (us; negative: a
+// loss), fitted on MI355X over N = 2048...11008, K = 4096...13824, 17 to 64
+// rows.  The halves have half the row blocks to sum, store and read back and
+// half the sharers per tile, which is worth S; their runs are twice as long,
+// and a granule of one or two row blocks costs more than half a granule of two
+// to four, which costs p per granule of the uncut run.  S jumps where the last
+// arrival of the uncut launch would fetch its sharers in more than one round
+// (more than 8).  E.g. M = 64, N = K = 4096 (8 sharers, 8 granules): 12.9 ->
+// 10.2 us; N = 2048: 14.9 -> 8.5; 8192 x 8192 (4 sharers, 32 granules): 20.0
+// -> 19.5; M = 48 there 17.1 -> 19.1 (not cut).
+double halves_gain(int rows, int wpt, int gpb) {
+  const int mb = ceil_div(rows, 16);
+  const bool rounds = wpt > 8;
+  const double p = 0.06;
+  double s;
+  if (mb <= 2)
+    s = rounds ? 2.8 : 1.0 + 0.045 * (rows - 16);
+  else if (mb == 3)
+    s = rounds ? 4.0 : 1.0 + 0.027 * (rows - 33);
+  else
+    s = rounds ? 6.5 : 3.2;
+  return s - p * gpb;
+}
+
 // Fitted time (us) of the streaming kernel: a pass over 49-64 rows takes
 // 12.1 + 0.285 per granule of the longest workgroup (N=K=4096: 8 granules,
 // 13.9; N=11008, K=4096 or 8192^2: 32, 20.3-21.2; N=28672, K=8192: 128, 48),
@@ -298,6 +326,8 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   pl.ksplit = 1;
   pl.tile_rows = 0;
   pl.partial_bytes = 0;
+  pl.row_halves = 1;
+  pl.half_rows = 0;
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
@@ -322,6 +352,20 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
     pl.sp.gpb = split.gpb;
     pl.sp.wpt = split.wpt;
     pl.sp.grid = split.wpt > 0 ? pl.sp.NT * split.wpt : ceil_div(pl.sp.NT * pl.sp.KG, split.gpb);
+    // Many rows and many workgroups per tile: cut the rows in two instead of
+    // the k range once more.  Each half is finished by half as many sharers,
+    // with half the rows to sum, store and read back.
+    const int half = 16 * ceil_div(ceil_div(rows, 2), 16);
+    const bool can = m <= kStreamMaxRows && half < rows && split.wpt >= 2 && cx.two_counters;
+    const bool want = cx.force.row_halves == 2 ||
+                      (cx.force.row_halves == 0 && halves_gain(rows, split.wpt, split.gpb) > 0.25);
+    if (can && want) {
+      pl.row_halves = 2;
+      pl.half_rows = half;
+      pl.sp.wpt = split.wpt / 2;
+      pl.sp.gpb = ceil_div(pl.sp.KG, pl.sp.wpt);
+      pl.sp.grid = pl.sp.NT * 2 * pl.sp.wpt;
+    }
   }
   pl.grid = pl.sp.grid;
   pl.launches = ceil_div(m, kStreamMaxRows);
@@ -329,7 +373,9 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   // partial-sum slot per workgroup (cut tiles) or two (runs that may start and
   // end inside a tile)
   const bool shared = pl.sp.wpt > 0 ? pl.sp.wpt > 1 : pl.sp.gpb % pl.sp.KG != 0;
-  if (shared) pl.partial_bytes = (size_t)stream_slots(pl.sp) * stream_slot_bytes(mb);
+  if (shared)
+    pl.partial_bytes = (size_t)stream_slots(pl.sp) *
+                       stream_slot_bytes(pl.row_halves == 2 ? pl.half_rows / 16 : mb);
   return pl;
 }
 
@@ -359,6 +405,8 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
     a.scratch = view.partials;
     a.gpb = 0;
     a.wpt = 0;
+    a.row_halves = 1;
+    a.half_rows = 0;
     // 128-row tiles: four waves with 128 x 128 accumulators; 64-row tiles: eight
     // waves with 64 x 64
     rc = pl.tile_rows == 128 ? launch_prefill_wide(a, groupsize != -1, pl.ksplit, stream)
@@ -378,6 +426,8 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
       a.scratch = view.partials;
       a.gpb = pl.sp.gpb;
       a.wpt = pl.sp.wpt;
+      a.row_halves = pl.row_halves;
+      a.half_rows = pl.half_rows;
       rc = launch_stream(a, groupsize != -1, pl.grid, stream);
     }
   }
@@ -439,7 +489,8 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   const int cus = device_cus(dev);
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0 && configure_device(dev)) {
-    const PlanCtx cx = {cus, use_static ? kStaticPartialBytes : kPoolPartialLimit, t_force};
+    PlanCtx cx = {cus, use_static ? kStaticPartialBytes : kPoolPartialLimit, t_force};
+    cx.two_counters = max_par >= 2;  // the counters of a tile sit min(max_par, 16) ints apart
     const Plan pl = make_plan(m, n, k, sms, cx);
     ScratchView view = {nullptr, nullptr};
     bool ok = true;
@@ -564,6 +615,8 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
 void marlin_amd_force_kernel(int which) { t_force.kernel = which == 1 || which == 2 ? which : 0; }
 
 void marlin_amd_force_k_slices(int slices) { t_force.k_slices = slices > 0 ? slices : 0; }
+
+void marlin_amd_force_row_halves(int mode) { t_force.row_halves = mode == 1 || mode == 2 ? mode : 0; }
 
 void marlin_amd_force_tile_rows(int rows) { t_force.tile_rows = rows == 64 || rows == 128 ? rows : 0; }
 

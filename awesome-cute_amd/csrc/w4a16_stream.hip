@@ -164,9 +164,23 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   const int wid = xcd_work_index((int)blockIdx.x, plan.grid);
   // my granules [u0, u1) of the tile-major sequence; my_tile = tile of u0
   int u0, u1, my_tile;
+  // One-tile form with the rows cut in two: work index w owns run w % wpt of
+  // (tile, half) number w / wpt; a half is a problem of its own (its rows of A
+  // and C, its ticket, its partial sums) over the same weights.
+  int vt = 0;        // (tile, half) number: my_tile * row_halves + half
+  int row0 = 0;      // first row of my half
+  int rows_m = p.M;  // rows of my half
   if constexpr (ONE_TILE) {
-    my_tile = wid / p.wpt;
-    const int run = wid - my_tile * p.wpt;
+    vt = wid / p.wpt;
+    const int run = wid - vt * p.wpt;
+    int half = 0;
+    my_tile = vt;
+    if (p.row_halves == 2) {
+      my_tile = vt >> 1;
+      half = vt & 1;
+      row0 = half * p.half_rows;
+      rows_m = half ? p.M - p.half_rows : p.half_rows;
+    }
     u0 = my_tile * KG + (run * KG) / p.wpt;
     u1 = my_tile * KG + ((run + 1) * KG) / p.wpt;
     if (my_tile >= plan.NT || u0 >= u1) return;
@@ -199,8 +213,8 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 #pragma unroll
   for (int i = 0; i < MB; i++) {
     int r = 16 * i + (kDmaA ? nu : (lane >> 2));
-    r = r < p.M ? r : p.M - 1;  // rows past M are never written back
-    a_lane[i] = r * p.K * 2 + 16 * ax;
+    r = r < rows_m ? r : rows_m - 1;  // rows past the end are never written back
+    a_lane[i] = (row0 + r) * p.K * 2 + 16 * ax;
   }
   char* lds_a = kDmaA ? smem + Lds::kRingBase + wave * Lds::kRingBytesPerWave
                       : smem + wave * (MB * 2048);
@@ -380,7 +394,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     // ticket knows every other partial has already landed in memory and reads
     // them with device-scope loads.  (Keeping a second, write-back copy in the
     // XCD's L2 for the reader was measured and dropped: 0.15 us slower.)
-    const int bf = ONE_TILE ? t * p.wpt : tile_first_block(plan, t);
+    const int bf = ONE_TILE ? vt * p.wpt : tile_first_block(plan, t);
     const int bl = ONE_TILE ? bf + p.wpt - 1 : tile_last_block(plan, t);
     bool writer = true;
     if (bl > bf) {
@@ -391,7 +405,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       const int mine = slot_of(wid) * part_bytes;
 #pragma unroll
       for (int i = 0; i < MB; i++)
-        if (16 * i + nu < p.M) {
+        if (16 * i + nu < rows_m) {
 #pragma unroll
           for (int h = 0; h < 2; h++) {
             const int at = (((i * 4 + wave) * 2 + h) * 64 + lane) * 16;
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
       __syncthreads();
       if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride], 1, __ATOMIC_RELAXED,
+        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride + (vt & (p.row_halves - 1))], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       writer = (s_ticket == bl - bf);
@@ -414,7 +428,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
         for (int b0 = bf; b0 <= bl; b0 += 8) {
           f4 v[2][8][2];
           auto fetch = [&](int i, f4 (&dst)[8][2]) {
-            const int at = ((((i * 4 + wave) * 2) * 64 + lane) * 16) | (16 * i + nu < p.M ? 0 : kOob);
+            const int at = ((((i * 4 + wave) * 2) * 64 + lane) * 16) | (16 * i + nu < rows_m ? 0 : kOob);
 #pragma unroll
             for (int u = 0; u < 8; u++) {
               const int b = b0 + u;
@@ -447,7 +461,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           res[i][1] = sum[i][1];
         }
         if (tid == 0)  // counters are handed back zeroed
-          __hip_atomic_store(&p.locks[t * p.lock_stride], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(&p.locks[t * p.lock_stride + (vt & (p.row_halves - 1))], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();  // s_ticket is reused by the next tile
     }
@@ -468,11 +482,11 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 #pragma unroll
         for (int i = 0; i < MB; i++) {
           const int m = 16 * i + nu;
-          if (m < p.M) {
+          if (m < rows_m) {
             h4 o = {(half_t)res[i][h][0], (half_t)res[i][h][1], (half_t)res[i][h][2],
                     (half_t)res[i][h][3]};
             if (!GROUP) o *= sc;
-            *(h4*)(C + (size_t)m * p.N + n0) = o;
+            *(h4*)(C + (size_t)(row0 + m) * p.N + n0) = o;
           }
         }
       }
@@ -492,9 +506,10 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       ikq += 4;
     }
     if constexpr (DEPTH == 2 && !kDmaA) {
-      // At most two granules per wave and both are already requested: a rolled
-      // loop over one copy of the compute code; the second granule moves into
-      // the first's registers in between.
+      // At most two granules per wave (the host picks this instance for no
+      // other run) and both are already requested: a rolled loop over one copy
+      // of the compute code; the second granule moves into the first's
+      // registers in between.
 #pragma unroll 1
       for (int i = 0; i < n_mine; i++) {
         compute(0);
@@ -581,11 +596,14 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
 // faster than four for every row-block count (M=16: N=11008 10.3 -> 9.9 us,
 // K=11008 10.4 -> 9.6; 64 rows at K=11008 21.2 -> 18.4), and eight slower
 // still: the more requests a CU has in flight, the slower the stream.  With
-// two row blocks two are better again (M=32, N=11008: 12.7 -> 12.4 us), with
-// three and four they are 2-5 % worse.
+// two row blocks on the LDS ring two are better again (M=32, N=11008:
+// 12.7 -> 12.4 us), with three and four they are 2-5 % worse.  In the one-tile
+// form the deep variant is never two deep: there the two-slot instance is the
+// rolled loop for waves that see at most two granules (see the kernel), which
+// launch_form below only picks for such runs.
 template <int MB, bool ONE_TILE>
 constexpr int deep_ring() {
-  return MB == 2 ? 2 : 3;
+  return MB == 2 && !ONE_TILE ? 2 : 3;
 }
 
 template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
@@ -638,7 +656,8 @@ static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
 }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream) {
-  const int mb = ceil_div(a.M, 16);
+  // row blocks per workgroup: of all rows, or of the larger half
+  const int mb = a.wpt > 0 && a.row_halves == 2 ? a.half_rows / 16 : ceil_div(a.M, 16);
   switch (mb * 2 + (group ? 1 : 0)) {
     case 2: return launch_one<1, false>(a, grid, stream);
     case 3: return launch_one<1, true>(a, grid, stream);

@@ -43,6 +43,8 @@ _lib.marlin_amd_force_k_slices.restype = None
 _lib.marlin_amd_force_k_slices.argtypes = [_I]
 _lib.marlin_amd_force_tile_rows.restype = None
 _lib.marlin_amd_force_tile_rows.argtypes = [_I]
+_lib.marlin_amd_force_row_halves.restype = None
+_lib.marlin_amd_force_row_halves.argtypes = [_I]
 _lib.marlin_amd_force_kernel.restype = None
 _lib.marlin_amd_force_kernel.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
@@ -278,6 +280,12 @@ def force_k_slices(slices):
 def force_tile_rows(rows):
     """Rows of C per prefill workgroup (64 or 128); 0 = choose by cost (calling thread only)."""
     _lib.marlin_amd_force_tile_rows(int(rows))
+
+
+def force_row_halves(mode):
+    """Whether the streaming kernel cuts 17..64 rows into two halves computed by separate
+    workgroups: 0 = choose by cost, 1 = never, 2 = wherever possible (calling thread only)."""
+    _lib.marlin_amd_force_row_halves(int(mode))
 
 
 def work_order(grid):

@@ -63,6 +63,14 @@ void marlin_amd_force_kernel(int which);
 void marlin_amd_force_k_slices(int slices);
 
 /*
+ * Whether the streaming kernel cuts 17..64 rows into two halves that separate
+ * workgroups compute (instead of cutting the k range of a tile once more), for
+ * the calling thread: 0 = choose by cost (default), 1 = never, 2 = wherever
+ * possible.  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_row_halves(int mode);
+
+/*
  * Rows of C per workgroup of the prefill kernel, for the calling thread: 0 =
  * choose by cost (default), 64 or 128.  No reference counterpart; for tests and tools.
  */

@@ -415,6 +415,51 @@ def test_four_wave_kernel_short_and_uneven_k_ranges(env, m, n, k, g, slices):
         marlin.force_k_slices(0)
 
 
+@pytest.mark.parametrize("groupsize", [128, -1])
+@pytest.mark.parametrize("m", [17, 32, 33, 48, 49, 64])
+def test_several_row_blocks_over_long_runs(env, m, groupsize):
+    """Two to four row blocks where every wave of the streaming kernel sees more
+    granules than its ring holds (the two-slot instance is only for runs of at
+    most two granules per wave; longer ones take the three-slot loop)."""
+    torch, marlin = env
+    for n, k in ((2048, 11008), (4096, 11008)):
+        rc, plan = marlin.plan(m, n, k, groupsize)
+        assert rc == 0 and plan["kernel"] == 1 and plan["granules_per_wg"] >= 9, plan
+        check(env, m, n, k, groupsize, seed=m + n)
+
+
+@pytest.mark.parametrize("groupsize", [128, -1])
+@pytest.mark.parametrize("m", [17, 18, 31, 32, 33, 40, 48, 49, 63, 64])
+def test_rows_cut_in_two_halves(env, m, groupsize):
+    """17 to 64 rows on the streaming kernel, whole and cut into two halves that
+    separate workgroups compute (each half its own ticket and partial sums):
+    both within the tolerance of the oracle, C written everywhere (it starts at
+    9), the same bits on a second call; the smallest legal workspace (one
+    counter per tile) has no room for the second ticket and is never cut."""
+    torch, marlin = env
+    marlin.force_kernel(1)
+    try:
+        for n, k in ((512, 2048), (2048, 4096), (1280, 1152)):
+            A, q, s, B, sp = O.make_problem(m, n, k, groupsize, seed=m + n)
+            ref = O.gemm(A, B, sp, n, groupsize)
+            for mode in (1, 2):
+                marlin.force_row_halves(mode)
+                rc, plan = marlin.plan(m, n, k, groupsize)
+                assert rc == 0 and plan["kernel"] == 1
+                c1 = gpu_gemm(env, A, B, sp, n, C_fill=9.0)
+                c2 = gpu_gemm(env, A, B, sp, n, C_fill=9.0)
+                assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
+                r = O.compare(c1, ref)
+                assert r.max_abs_err <= TOL * r.max_abs_ref, (mode, n, k, r.max_abs_err)
+                assert r.rel_mean_abs_err <= REL_MEAN_TOL
+            c3 = gpu_gemm(env, A, B, sp, n, max_par=1, C_fill=9.0)  # mode 2 still set
+            r = O.compare(c3, ref)
+            assert r.max_abs_err <= TOL * r.max_abs_ref
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_row_halves(0)
+
+
 @pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
 def test_frozen_known_answers(env, tag, groupsize):
     """The committed known answers (tests/golden): dequantised weights bit for
