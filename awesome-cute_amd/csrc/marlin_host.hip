@@ -292,13 +292,16 @@ double halves_gain(int rows, int wpt, int gpb) {
   return s - p * gpb;
 }
 
-// Fitted time (us) of the streaming kernel: a pass over 49-64 rows takes
-// 12.1 + 0.285 per granule of the longest workgroup (N=K=4096: 8 granules,
-// 13.9; N=11008, K=4096 or 8192^2: 32, 20.3-21.2; N=28672, K=8192: 128, 48),
-// fewer rows a share of that, up to 16 rows 5.1 + 0.16 per granule.
+// Fitted time (us) of the streaming kernel with uncut rows: a pass over 49-64
+// rows takes 11.3 + 0.28 per granule of the longest workgroup (N=K=4096: 8
+// granules, 12.9; N=8192, K=4096: 16, 15.5; N=4096, K=11008: 22, 18.0;
+// N=11008, K=4096 or 8192^2: 32, 18.5-20; N=28672, K=8192: 128, 46), fewer
+// rows a share of that, up to 16 rows 5.1 + 0.16 per granule; every launch
+// after the first waits a microsecond for the one before (65 rows at N=4096,
+// K=11008: 18.0 + 9.0 alone, 27.0 in a row).
 double stream_cost(int m, int n, int k, int cus) {
   const StreamSplit s4 = choose_stream_split(4, n, k, cus);
-  const double full = 12.1 + 0.285 * s4.gpb + (s4.straddle ? 11.0 : 0.0);
+  const double full = 11.3 + 0.28 * s4.gpb + (s4.straddle ? 11.0 : 0.0);
   const int tail = m % kStreamMaxRows;
   double t = (m / kStreamMaxRows) * full;
   if (tail > 16) {
@@ -307,13 +310,20 @@ double stream_cost(int m, int n, int k, int cus) {
     const StreamSplit s1 = choose_stream_split(1, n, k, cus);
     t += 5.1 + 0.16 * s1.gpb + (s1.straddle ? 3.5 : 0.0);
   }
-  return t;
+  return t + 1.0 * (ceil_div(m, kStreamMaxRows) - 1);
 }
 
 bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   // no measurement favours 64-row prefill tiles below four row blocks
   if (m <= 48) return false;
-  return prefill_cost(m, n, k, cx) <= stream_cost(m, n, k, cx.cus);
+  double stream = stream_cost(m, n, k, cx.cus);
+  if (m <= kStreamMaxRows && cx.force.row_halves != 1 && cx.two_counters) {
+    // what the launch gains where make_plan cuts its rows in two
+    const StreamSplit split = choose_stream_split(ceil_div(m, 16), n, k, cx.cus);
+    const double gain = split.wpt >= 2 ? halves_gain(m, split.wpt, split.gpb) : 0.0;
+    if (gain > 0.25) stream -= gain;
+  }
+  return prefill_cost(m, n, k, cx) <= stream;
 }
 
 Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
@@ -386,8 +396,9 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
             hipStream_t stream) {
   // the caller's workspace holds at least n/128 * max_par zero ints
   // (reference marlin_gemm.cpp:29-31, marlin_cute_kernel.cu:68); one counter
-  // per column tile is used, and the counters are spread max_par ints apart
-  // (64 bytes at the launcher's default of 16)
+  // per column tile is used (two where the rows are cut in halves: the plan
+  // only does that when max_par >= 2), and the counters are spread max_par
+  // ints apart (64 bytes at the launcher's default of 16)
   const int lock_stride = max_par > 16 ? 16 : max_par;
   (void)hipGetLastError();  // an earlier call's error is not this launch's
   int rc = MARLIN_OK;
