@@ -129,8 +129,9 @@ constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (
 // which a workgroup never leaves its tile: no tile bookkeeping in the main
 // loop and exactly one finish at the end.  Otherwise the first form (equal
 // runs of the tile-major sequence), where a run may cross tile boundaries.
-template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
+template <int MB, bool GROUP, int DEPTH, bool ONE_TILE, bool HALVES>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
+  static_assert(!HALVES || (ONE_TILE && MB <= 2), "rows are only cut in the one-tile form");
   extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH, ONE_TILE>::kBytes
   __shared__ int s_ticket;
   using Lds = StreamLds<MB, DEPTH, ONE_TILE>;
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     int* l_ = p.locks;
     float* sc_ = p.scratch;
     asm volatile("" ::"s"(a_), "s"(b_), "s"(s_), "s"(c_), "s"(l_), "s"(sc_), "s"(p.M), "s"(p.N),
-                 "s"(p.K), "s"(p.gpb), "s"(p.wpt), "s"(p.lock_stride));
+                 "s"(p.K), "s"(p.gpb), "s"(p.wpt), "s"(p.lock_stride), "s"(p.half_rows));
   }
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     const int run = wid - vt * p.wpt;
     int half = 0;
     my_tile = vt;
-    if (p.row_halves == 2) {
+    if constexpr (HALVES) {
       my_tile = vt >> 1;
       half = vt & 1;
       row0 = half * p.half_rows;
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
       __syncthreads();
       if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride + (vt & (p.row_halves - 1))], 1, __ATOMIC_RELAXED,
+        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride + (HALVES ? (vt & 1) : 0)], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       writer = (s_ticket == bl - bf);
@@ -461,7 +462,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           res[i][1] = sum[i][1];
         }
         if (tid == 0)  // counters are handed back zeroed
-          __hip_atomic_store(&p.locks[t * p.lock_stride + (vt & (p.row_halves - 1))], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(&p.locks[t * p.lock_stride + (HALVES ? (vt & 1) : 0)], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();  // s_ticket is reused by the next tile
     }
@@ -610,10 +611,15 @@ template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
 static int configure_variant() {
   constexpr int lds = StreamLds<MB, DEPTH, ONE_TILE>::kBytes;
   if (lds <= 65536) return 0;  // within the default limit of dynamic LDS
-  return hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, ONE_TILE>,
-                             hipFuncAttributeMaxDynamicSharedMemorySize, lds) == hipSuccess
-             ? 0
-             : 3;
+  if (hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, ONE_TILE, false>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+    return 3;
+  if constexpr (ONE_TILE && MB <= 2) {
+    if (hipFuncSetAttribute((const void*)stream_kernel<MB, GROUP, DEPTH, ONE_TILE, true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return 3;
+  }
+  return 0;
 }
 template <int MB, bool ONE_TILE>
 static int configure_form() {
@@ -636,8 +642,17 @@ int configure_stream_kernels() {
 template <int MB, bool GROUP, int DEPTH, bool ONE_TILE>
 static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
   constexpr int lds = StreamLds<MB, DEPTH, ONE_TILE>::kBytes;
-  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE>), dim3(grid), dim3(256), lds,
-                     stream, a);
+  // (the instance with the rows cut in two is a kernel of its own, so that
+  // launches that do not cut them carry none of its bookkeeping)
+  if constexpr (ONE_TILE && MB <= 2) {
+    if (a.row_halves == 2) {
+      hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE, true>), dim3(grid), dim3(256),
+                         lds, stream, a);
+      return launch_status();
+    }
+  }
+  hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE, false>), dim3(grid), dim3(256),
+                     lds, stream, a);
   return launch_status();
 }
 
