@@ -124,8 +124,8 @@ struct Plan {
   int ksplit;            // prefill: slices of the k range per tile
   int tile_rows;         // prefill: rows of C per workgroup
   size_t partial_bytes;  // fp32 partial sums the launch exchanges through scratch (0: none)
-  int row_halves;        // streaming, one-tile form: 2 when the rows are cut into two halves
-  int half_rows;         // rows of the first half
+  int row_parts;         // streaming, one-tile form: parts the rows are cut into (1: uncut)
+  int part_rows;         // rows of a part (the last one has the rest)
 };
 
 constexpr int kStreamMaxRows = 64;
@@ -146,7 +146,7 @@ struct PlanCtx {
   int cus;
   size_t partial_limit;
   Force force;
-  bool two_counters = true;  // the workspace has room for two counters per column tile
+  int counters = 16;  // ints of the workspace per column tile: min(max_par, 16)
 };
 
 // Cost in us of the prefill kernel with `tiles` tiles of tile_rows rows cut into
@@ -313,16 +313,43 @@ double stream_cost(int m, int n, int k, int cus) {
   return t + 1.0 * (ceil_div(m, kStreamMaxRows) - 1);
 }
 
+// More than 64 rows in one streaming launch: the rows cut into parts of 32,
+// every (tile, part) a problem of its own for wpt workgroups.  Possible while
+// there is a CU per (tile, part) and a counter per part; costs what a 32-row
+// launch of that split costs (0.65 of the fit above; measured 12.6 us against
+// 13.2 for M = 128 at N = K = 4096, 22.9 / 23.0 at K = 11008, 17.1 / 17.0 for
+// M = 256 with one workgroup per tile and part).  Sets wpt
+// and the granules per run; returns the cost in us, or a negative number where
+// it cannot be done.
+double stream_parts_cost(int m, int n, int k, const PlanCtx& cx, int* parts, int* wpt, int* gpb) {
+  const int NT = n / kTileN, KG = k / kGranuleK;
+  const int P = ceil_div(m, 32);
+  if (m <= kStreamMaxRows || P > cx.counters || NT * P > cx.cus || cx.force.row_halves == 1)
+    return -1.0;
+  int w = cx.cus / (NT * P);
+  if (w > KG) w = KG;
+  // more than 8 sharers would be fetched in two rounds by the last arrival
+  if (w > 8) w = 8;
+  *parts = P;
+  *wpt = w;
+  *gpb = ceil_div(KG, w);
+  // (a launch that exchanges nothing saves the 2 us the fit holds for that)
+  return 0.65 * (11.3 + 0.28 * *gpb) - (w == 1 ? 2.0 : 0.0);
+}
+
 bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   // no measurement favours 64-row prefill tiles below four row blocks
   if (m <= 48) return false;
   double stream = stream_cost(m, n, k, cx.cus);
-  if (m <= kStreamMaxRows && cx.force.row_halves != 1 && cx.two_counters) {
+  if (m <= kStreamMaxRows && cx.force.row_halves != 1 && cx.counters >= 2) {
     // what the launch gains where make_plan cuts its rows in two
     const StreamSplit split = choose_stream_split(ceil_div(m, 16), n, k, cx.cus);
     const double gain = split.wpt >= 2 ? halves_gain(m, split.wpt, split.gpb) : 0.0;
     if (gain > 0.25) stream -= gain;
   }
+  int parts, wpt, gpb;
+  const double cut = stream_parts_cost(m, n, k, cx, &parts, &wpt, &gpb);
+  if (cut > 0.0 && cut < stream) stream = cut;
   return prefill_cost(m, n, k, cx) <= stream;
 }
 
@@ -336,8 +363,8 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   pl.ksplit = 1;
   pl.tile_rows = 0;
   pl.partial_bytes = 0;
-  pl.row_halves = 1;
-  pl.half_rows = 0;
+  pl.row_parts = 1;
+  pl.part_rows = 0;
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
@@ -353,6 +380,25 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   pl.kernel = 1;
   const int rows = m < kStreamMaxRows ? m : kStreamMaxRows;
   const int mb = ceil_div(rows, 16);
+  {
+    // more than 64 rows: one launch with the rows cut into parts of 32 where
+    // that is cheaper than a launch per 64 rows
+    int parts = 0, wpt = 0, gpb = 0;
+    const double cut = sms > 0 ? -1.0 : stream_parts_cost(m, n, k, cx, &parts, &wpt, &gpb);
+    if (cut > 0.0 && (cx.force.row_halves == 2 || cut < stream_cost(m, n, k, cx.cus))) {
+      pl.sp.NT = n / kTileN;
+      pl.sp.KG = k / kGranuleK;
+      pl.sp.gpb = gpb;
+      pl.sp.wpt = wpt;
+      pl.sp.grid = pl.sp.NT * parts * wpt;
+      pl.row_parts = parts;
+      pl.part_rows = 32;
+      pl.grid = pl.sp.grid;
+      pl.launches = 1;
+      if (wpt > 1) pl.partial_bytes = (size_t)stream_slots(pl.sp) * stream_slot_bytes(2);
+      return pl;
+    }
+  }
   if (sms > 0) {
     pl.sp = make_stream_plan(n, k, sms > kMaxStreamGrid ? kMaxStreamGrid : sms);
   } else {
@@ -366,12 +412,12 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
     // the k range once more.  Each half is finished by half as many sharers,
     // with half the rows to sum, store and read back.
     const int half = 16 * ceil_div(ceil_div(rows, 2), 16);
-    const bool can = m <= kStreamMaxRows && half < rows && split.wpt >= 2 && cx.two_counters;
+    const bool can = m <= kStreamMaxRows && half < rows && split.wpt >= 2 && cx.counters >= 2;
     const bool want = cx.force.row_halves == 2 ||
                       (cx.force.row_halves == 0 && halves_gain(rows, split.wpt, split.gpb) > 0.25);
     if (can && want) {
-      pl.row_halves = 2;
-      pl.half_rows = half;
+      pl.row_parts = 2;
+      pl.part_rows = half;
       pl.sp.wpt = split.wpt / 2;
       pl.sp.gpb = ceil_div(pl.sp.KG, pl.sp.wpt);
       pl.sp.grid = pl.sp.NT * 2 * pl.sp.wpt;
@@ -385,7 +431,7 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   const bool shared = pl.sp.wpt > 0 ? pl.sp.wpt > 1 : pl.sp.gpb % pl.sp.KG != 0;
   if (shared)
     pl.partial_bytes = (size_t)stream_slots(pl.sp) *
-                       stream_slot_bytes(pl.row_halves == 2 ? pl.half_rows / 16 : mb);
+                       stream_slot_bytes(pl.row_parts > 1 ? pl.part_rows / 16 : mb);
   return pl;
 }
 
@@ -416,20 +462,22 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
     a.scratch = view.partials;
     a.gpb = 0;
     a.wpt = 0;
-    a.row_halves = 1;
-    a.half_rows = 0;
+    a.row_parts = 1;
+    a.part_rows = 0;
     // 128-row tiles: four waves with 128 x 128 accumulators; 64-row tiles: eight
     // waves with 64 x 64
     rc = pl.tile_rows == 128 ? launch_prefill_wide(a, groupsize != -1, pl.ksplit, stream)
                              : launch_prefill(a, groupsize != -1, pl.ksplit, stream);
   } else {
-    for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += kStreamMaxRows) {
+    // a launch per 64 rows, or one launch over all rows cut into parts
+    const int rows_per_launch = pl.launches == 1 ? m : kStreamMaxRows;
+    for (int m0 = 0; m0 < m && rc == MARLIN_OK; m0 += rows_per_launch) {
       GemmArgs a;
       a.A = (const char*)A + (size_t)m0 * k * 2;
       a.B = B;
       a.C = (char*)C + (size_t)m0 * n * 2;
       a.S = s;
-      a.M = m - m0 < kStreamMaxRows ? m - m0 : kStreamMaxRows;
+      a.M = m - m0 < rows_per_launch ? m - m0 : rows_per_launch;
       a.N = n;
       a.K = k;
       a.locks = (int*)workspace;
@@ -437,8 +485,8 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
       a.scratch = view.partials;
       a.gpb = pl.sp.gpb;
       a.wpt = pl.sp.wpt;
-      a.row_halves = pl.row_halves;
-      a.half_rows = pl.half_rows;
+      a.row_parts = pl.row_parts;
+      a.part_rows = pl.part_rows;
       rc = launch_stream(a, groupsize != -1, pl.grid, stream);
     }
   }
@@ -501,7 +549,7 @@ int run(const void* A, const void* B, void* C, const void* s, int m, int n, int 
   rc = MARLIN_ERR_RUNTIME;
   if (cus > 0 && configure_device(dev)) {
     PlanCtx cx = {cus, use_static ? kStaticPartialBytes : kPoolPartialLimit, t_force};
-    cx.two_counters = max_par >= 2;  // the counters of a tile sit min(max_par, 16) ints apart
+    cx.counters = max_par > 16 ? 16 : max_par;  // the counters of a tile sit that many ints apart
     const Plan pl = make_plan(m, n, k, sms, cx);
     ScratchView view = {nullptr, nullptr};
     bool ok = true;
@@ -620,6 +668,8 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[7] = pl.tile_rows;
   out[8] = pl.kernel == 1 ? pl.sp.wpt : 0;
   out[9] = (int)(pl.partial_bytes >> 10);
+  out[10] = pl.kernel == 1 ? pl.row_parts : 1;
+  out[11] = pl.kernel == 1 ? pl.part_rows : 0;
   return rc;
 }
 

@@ -170,10 +170,11 @@ struct GemmArgs {
   float* scratch;   // partial sums of shared tiles (null if no tile is shared)
   int gpb;          // granules per workgroup (streaming kernel; the most, when wpt > 0)
   int wpt;          // workgroups per column tile, or 0 (see StreamPlan)
-  int row_halves;   // streaming kernel, wpt > 0: 1, or 2 when the rows are cut into two halves
-                    // of `half_rows` that separate workgroups compute (wpt workgroups per
-                    // column tile and half; needs lock_stride >= 2)
-  int half_rows;    // rows of the first half (a multiple of 16)
+  int row_parts;    // streaming kernel, wpt > 0: 1, or the number of parts the rows are cut
+                    // into, `part_rows` each (the last one the rest), that separate
+                    // workgroups compute: wpt workgroups per column tile and part; needs
+                    // lock_stride >= row_parts
+  int part_rows;    // rows of a part: 16 or 32
 };
 
 // bytes of fp32 partial sums of mb row blocks of 16 (one slot)

@@ -129,9 +129,9 @@ constexpr int wait_vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | (
 // which a workgroup never leaves its tile: no tile bookkeeping in the main
 // loop and exactly one finish at the end.  Otherwise the first form (equal
 // runs of the tile-major sequence), where a run may cross tile boundaries.
-template <int MB, bool GROUP, int DEPTH, bool ONE_TILE, bool HALVES>
+template <int MB, bool GROUP, int DEPTH, bool ONE_TILE, bool PARTS>
 __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
-  static_assert(!HALVES || (ONE_TILE && MB <= 2), "rows are only cut in the one-tile form");
+  static_assert(!PARTS || (ONE_TILE && MB <= 2), "rows are only cut in the one-tile form, into parts of 16 or 32");
   extern __shared__ __attribute__((aligned(16))) char smem[];  // StreamLds<MB, DEPTH, ONE_TILE>::kBytes
   __shared__ int s_ticket;
   using Lds = StreamLds<MB, DEPTH, ONE_TILE>;
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
     int* l_ = p.locks;
     float* sc_ = p.scratch;
     asm volatile("" ::"s"(a_), "s"(b_), "s"(s_), "s"(c_), "s"(l_), "s"(sc_), "s"(p.M), "s"(p.N),
-                 "s"(p.K), "s"(p.gpb), "s"(p.wpt), "s"(p.lock_stride), "s"(p.half_rows));
+                 "s"(p.K), "s"(p.gpb), "s"(p.wpt), "s"(p.lock_stride), "s"(p.row_parts), "s"(p.part_rows));
   }
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
@@ -165,22 +165,22 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
   const int wid = xcd_work_index((int)blockIdx.x, plan.grid);
   // my granules [u0, u1) of the tile-major sequence; my_tile = tile of u0
   int u0, u1, my_tile;
-  // One-tile form with the rows cut in two: work index w owns run w % wpt of
-  // (tile, half) number w / wpt; a half is a problem of its own (its rows of A
-  // and C, its ticket, its partial sums) over the same weights.
-  int vt = 0;        // (tile, half) number: my_tile * row_halves + half
-  int row0 = 0;      // first row of my half
-  int rows_m = p.M;  // rows of my half
+  // One-tile form with the rows cut into parts: work index w owns run w % wpt
+  // of (tile, part) number w / wpt; a part is a problem of its own (its rows of
+  // A and C, its ticket, its partial sums) over the same weights.
+  int vt = 0;        // (tile, part) number: my_tile * row_parts + part
+  int part = 0;
+  int row0 = 0;      // first row of my part
+  int rows_m = p.M;  // rows of my part
   if constexpr (ONE_TILE) {
     vt = wid / p.wpt;
     const int run = wid - vt * p.wpt;
-    int half = 0;
     my_tile = vt;
-    if constexpr (HALVES) {
-      my_tile = vt >> 1;
-      half = vt & 1;
-      row0 = half * p.half_rows;
-      rows_m = half ? p.M - p.half_rows : p.half_rows;
+    if constexpr (PARTS) {
+      my_tile = vt / p.row_parts;
+      part = vt - my_tile * p.row_parts;
+      row0 = part * p.part_rows;
+      rows_m = min(p.part_rows, p.M - row0);
     }
     u0 = my_tile * KG + (run * KG) / p.wpt;
     u1 = my_tile * KG + ((run + 1) * KG) / p.wpt;
@@ -416,7 +416,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
       __builtin_amdgcn_s_waitcnt(kWaitVm0);  // my stores have been acknowledged
       __syncthreads();
       if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride + (HALVES ? (vt & 1) : 0)], 1, __ATOMIC_RELAXED,
+        s_ticket = __hip_atomic_fetch_add(&p.locks[t * p.lock_stride + part], 1, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       writer = (s_ticket == bl - bf);
@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256) void stream_kernel(GemmArgs p) {
           res[i][1] = sum[i][1];
         }
         if (tid == 0)  // counters are handed back zeroed
-          __hip_atomic_store(&p.locks[t * p.lock_stride + (HALVES ? (vt & 1) : 0)], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(&p.locks[t * p.lock_stride + part], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       __syncthreads();  // s_ticket is reused by the next tile
     }
@@ -645,7 +645,7 @@ static int launch_variant(const GemmArgs& a, int grid, hipStream_t stream) {
   // (the instance with the rows cut in two is a kernel of its own, so that
   // launches that do not cut them carry none of its bookkeeping)
   if constexpr (ONE_TILE && MB <= 2) {
-    if (a.row_halves == 2) {
+    if (a.row_parts > 1) {
       hipLaunchKernelGGL((stream_kernel<MB, GROUP, DEPTH, ONE_TILE, true>), dim3(grid), dim3(256),
                          lds, stream, a);
       return launch_status();
@@ -671,8 +671,8 @@ static int launch_one(const GemmArgs& a, int grid, hipStream_t stream) {
 }
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream) {
-  // row blocks per workgroup: of all rows, or of the larger half
-  const int mb = a.wpt > 0 && a.row_halves == 2 ? a.half_rows / 16 : ceil_div(a.M, 16);
+  // row blocks per workgroup: of all rows, or of a part
+  const int mb = a.wpt > 0 && a.row_parts > 1 ? a.part_rows / 16 : ceil_div(a.M, 16);
   switch (mb * 2 + (group ? 1 : 0)) {
     case 2: return launch_one<1, false>(a, grid, stream);
     case 3: return launch_one<1, true>(a, grid, stream);

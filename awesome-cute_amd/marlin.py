@@ -283,8 +283,9 @@ def force_tile_rows(rows):
 
 
 def force_row_halves(mode):
-    """Whether the streaming kernel cuts 17..64 rows into two halves computed by separate
-    workgroups: 0 = choose by cost, 1 = never, 2 = wherever possible (calling thread only)."""
+    """Whether the streaming kernel cuts the rows into parts computed by separate workgroups
+    (17..64 rows in two halves, more in parts of 32 within one launch): 0 = choose by cost,
+    1 = never, 2 = wherever possible (calling thread only)."""
     _lib.marlin_amd_force_row_halves(int(mode))
 
 
@@ -297,10 +298,10 @@ def work_order(grid):
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     """Kernel, grid and stream-K partition marlin_gemm would use."""
-    out = (ctypes.c_int * 10)()
+    out = (ctypes.c_int * 12)()
     rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
     keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
-            "k_slices", "tile_rows", "wgs_per_tile", "partial_kib")
+            "k_slices", "tile_rows", "wgs_per_tile", "partial_kib", "row_parts", "part_rows")
     return rc, dict(zip(keys, out))
 
 

@@ -29,8 +29,10 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * column tile when the streaming kernel cuts every tile into that many runs
  * (then out[2] is the longest run), 0 when it cuts the tile-major sequence of
  * granules into equal runs of out[2]; out[9] = KiB of partial sums the launch
- * exchanges through the library's scratch (0 = none).  `out` holds 10 ints.
- * Returns the marlin_gemm error code for the shape.
+ * exchanges through the library's scratch (0 = none); out[10] = parts the
+ * streaming kernel cuts the rows into (1 = uncut; every part is a problem of
+ * its own for out[8] workgroups per column tile), out[11] = rows of a part.
+ * `out` holds 12 ints.  Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int *out);
@@ -63,10 +65,12 @@ void marlin_amd_force_kernel(int which);
 void marlin_amd_force_k_slices(int slices);
 
 /*
- * Whether the streaming kernel cuts 17..64 rows into two halves that separate
- * workgroups compute (instead of cutting the k range of a tile once more), for
- * the calling thread: 0 = choose by cost (default), 1 = never, 2 = wherever
- * possible.  No reference counterpart; for tests and tools.
+ * Whether the streaming kernel cuts the rows into parts that separate
+ * workgroups compute (17..64 rows into two halves instead of cutting the k
+ * range of a tile once more; more than 64 rows into parts of 32 in one launch
+ * instead of a launch per 64 rows), for the calling thread: 0 = choose by cost
+ * (default), 1 = never, 2 = wherever possible.  No reference counterpart; for
+ * tests and tools.
  */
 void marlin_amd_force_row_halves(int mode);
 

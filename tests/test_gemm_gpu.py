@@ -460,6 +460,40 @@ def test_rows_cut_in_two_halves(env, m, groupsize):
         marlin.force_row_halves(0)
 
 
+@pytest.mark.parametrize("groupsize", [128, -1])
+@pytest.mark.parametrize("m", [65, 96, 100, 128, 129, 200, 256, 300, 511])
+def test_more_than_64_rows_in_one_streaming_launch(env, m, groupsize):
+    """More than 64 rows on the streaming kernel as one launch whose rows are
+    cut into parts of 32, every (column tile, part) with its own workgroups,
+    ticket and partial sums -- where there is a CU per (tile, part) and a
+    counter per part in the workspace; otherwise a launch per 64 rows.  Against
+    the oracle, C written everywhere, the same bits twice."""
+    torch, marlin = env
+    marlin.force_kernel(1)
+    marlin.force_row_halves(2)
+    try:
+        for n, k, max_par in ((512, 2048, 16), (1024, 1152, 16), (256, 4096, 16), (512, 1024, 4),
+                              (512, 1024, 1)):
+            parts = -(-m // 32)
+            fits = parts <= min(max_par, 16) and (n // 128) * parts <= 256
+            rc, plan = marlin.plan(m, n, k, groupsize)
+            assert rc == 0 and plan["kernel"] == 1
+            if max_par == 16:
+                assert plan["launches"] == (1 if fits else -(-m // 64)), plan
+                assert plan["row_parts"] == (parts if fits else 1)
+            A, q, s, B, sp = O.make_problem(m, n, k, groupsize, seed=m + n + max_par)
+            ref = O.gemm(A, B, sp, n, groupsize)
+            c1 = gpu_gemm(env, A, B, sp, n, max_par=max_par, C_fill=9.0)
+            c2 = gpu_gemm(env, A, B, sp, n, max_par=max_par, C_fill=9.0)
+            assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
+            r = O.compare(c1, ref)
+            assert r.max_abs_err <= TOL * r.max_abs_ref, (n, k, max_par, r.max_abs_err)
+            assert r.rel_mean_abs_err <= REL_MEAN_TOL
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_row_halves(0)
+
+
 @pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
 def test_frozen_known_answers(env, tag, groupsize):
     """The committed known answers (tests/golden): dequantised weights bit for
@@ -709,9 +743,9 @@ def test_scratch_is_sized_by_the_plan_and_can_be_released(env):
     assert marlin.scratch_bytes(0)[1] == 8
     # growth on one stream: a sliced prefill launch needs more than decode did
     with torch.cuda.stream(streams[0]):
-        rc, plan = marlin.plan(256, 4096, 4096, 128)
+        rc, plan = marlin.plan(512, 4096, 4096, 128)
         assert plan["k_slices"] > 1 and plan["partial_kib"] > 4096
-        check(env, 256, 4096, 4096, 128, seed=6)
+        check(env, 512, 4096, 4096, 128, seed=6)
         held, bufs = marlin.scratch_bytes(0)
         assert bufs == 9  # the smaller buffer stays until release (graphs may name it)
         assert held <= 8 * (4 * MiB + 65536) + 2 * plan["partial_kib"] * 1024 + 65536 + MiB
@@ -800,20 +834,26 @@ def test_random_shapes_kernels_and_knobs(env, seed):
 @pytest.mark.parametrize("m,n,k,g", [(128, 4096, 11008, 128), (160, 4096, 11008, -1),
                                      (96, 5120, 13568, 128), (320, 4096, 11008, 128)])
 def test_mid_rows_deep_k_planned_slices(env, m, n, k, g):
-    """Between decode and prefill over a deep k range the host cuts the tiles
-    into more than four k slices (or three, not a power of two); oracle on a
-    column slice, GPU on the whole shape, and twice the same bits."""
+    """Between decode and prefill over a deep k range the prefill kernel's
+    tiles are cut into more than four k slices (or three, not a power of two)
+    by the host's cost model (the kernel is pinned: some of these shapes stream
+    with their rows in parts otherwise); oracle on a column slice, GPU on the
+    whole shape, and twice the same bits."""
     torch, marlin = env
-    rc, plan = marlin.plan(m, n, k, g)
-    assert rc == 0 and plan["kernel"] == 2 and plan["k_slices"] in (3, 5, 6), plan
-    A, q, s, B, sp = O.make_problem(m, n, k, g, seed=m + k)
-    C = gpu_gemm(env, A, B, sp, n)
-    for c0 in (0, n - 256):
-        Bs = np.ascontiguousarray(B[:, 2 * c0:2 * (c0 + 256)])
-        ss = np.ascontiguousarray(sp[:, c0:c0 + 256])
-        r = O.compare(C[:, c0:c0 + 256], O.gemm(A, Bs, ss, 256, g))
-        assert r.max_abs_err <= TOL * r.max_abs_ref, (c0, r.max_abs_err, r.max_abs_ref)
-    assert np.array_equal(gpu_gemm(env, A, B, sp, n).view(np.uint16), C.view(np.uint16))
+    marlin.force_kernel(2)
+    try:
+        rc, plan = marlin.plan(m, n, k, g)
+        assert rc == 0 and plan["kernel"] == 2 and plan["k_slices"] in (3, 5, 6), plan
+        A, q, s, B, sp = O.make_problem(m, n, k, g, seed=m + k)
+        C = gpu_gemm(env, A, B, sp, n)
+        for c0 in (0, n - 256):
+            Bs = np.ascontiguousarray(B[:, 2 * c0:2 * (c0 + 256)])
+            ss = np.ascontiguousarray(sp[:, c0:c0 + 256])
+            r = O.compare(C[:, c0:c0 + 256], O.gemm(A, Bs, ss, 256, g))
+            assert r.max_abs_err <= TOL * r.max_abs_ref, (c0, r.max_abs_err, r.max_abs_ref)
+        assert np.array_equal(gpu_gemm(env, A, B, sp, n).view(np.uint16), C.view(np.uint16))
+    finally:
+        marlin.force_kernel(0)
 
 
 def test_config4_prefill_rows_sample(env):

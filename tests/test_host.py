@@ -210,13 +210,14 @@ def test_kernel_choice_by_cost(marlin):
     """Few rows go through the streaming kernel, many through the prefill
     kernel, whose k range is cut into slices (the cheapest count, at most eight)
     while tiles alone would leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
-    so do more rows while twice as many tiles save k slices.  The knobs override
-    the choice."""
+    so do more rows while twice as many tiles save k slices; up to a few hundred
+    rows over small weights stream in one launch with the rows cut into parts of
+    32.  The knobs override the choice."""
     for m, n, k, kernel, slices, rows in [
             (1, 4096, 4096, 1, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
-            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 2, 4, 64),
-            (128, 4096, 4096, 2, 4, 64), (512, 4096, 4096, 2, 2, 64),
-            (128, 4096, 11008, 2, 6, 64), (640, 4096, 11008, 2, 3, 128),
+            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 1, 1, 0),
+            (128, 4096, 4096, 1, 1, 0), (512, 4096, 4096, 2, 2, 64),
+            (128, 8192, 8192, 2, 4, 64), (640, 4096, 11008, 2, 3, 128),
             (512, 4096, 11008, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
             (1536, 4096, 4096, 2, 1, 128), (2048, 4096, 4096, 2, 1, 128)]:
         rc, p = marlin.plan(m, n, k, 128)
@@ -224,10 +225,18 @@ def test_kernel_choice_by_cost(marlin):
             (m, n, k, p)
         if kernel == 2:
             assert p["grid"] == -(-m // rows) * (n // 256) * slices
+    # rows in parts: one launch, a workgroup set per (tile, part)
+    rc, p = marlin.plan(128, 4096, 4096, 128)
+    assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 4, 32, 2)
+    assert p["grid"] == 32 * 4 * 2
+    rc, p = marlin.plan(64, 4096, 4096, 128)
+    assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 2, 32, 4)
+    rc, p = marlin.plan(16, 4096, 4096, 128)
+    assert (p["row_parts"], p["wgs_per_tile"]) == (1, 8)
     try:
         marlin.force_kernel(1)
         rc, p = marlin.plan(2048, 4096, 4096, 128)
-        assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32
+        assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32 and p["row_parts"] == 1
         marlin.force_kernel(2)
         rc, p = marlin.plan(100, 512, 1024, 128)
         assert rc == 0 and p["kernel"] == 2
@@ -381,9 +390,13 @@ def test_scratch_accounting_and_plan_sizes_without_gpu(marlin):
     assert p["kernel"] == 1 and p["partial_kib"] == 0
     rc, p = marlin.plan(2048, 4096, 4096, 128)
     assert p["kernel"] == 2 and p["k_slices"] == 1 and p["partial_kib"] == 0
-    rc, p = marlin.plan(256, 4096, 4096, 128)
+    rc, p = marlin.plan(512, 4096, 4096, 128)
     assert p["kernel"] == 2 and p["k_slices"] > 1
     assert p["partial_kib"] == p["grid"] * p["tile_rows"] * 256 * 4 // 1024
+    rc, p = marlin.plan(128, 4096, 4096, 128)  # rows in parts of 32: two row blocks per slot
+    assert p["kernel"] == 1 and p["row_parts"] == 4 and p["partial_kib"] == 2 * p["grid"] * 2 * 8
+    rc, p = marlin.plan(256, 4096, 4096, 128)  # a workgroup per tile and part: no exchange
+    assert p["kernel"] == 1 and p["wgs_per_tile"] == 1 and p["partial_kib"] == 0
     assert marlin._lib.marlin_gemm_static_capacity() == 32 << 20
 
 
