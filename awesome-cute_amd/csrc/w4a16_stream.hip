@@ -1,7 +1,9 @@
-// Streaming W4A16 kernel for at most 64 activation rows per launch (decode and
-// small batch): the weight stream is the roofline, so every wave keeps a ring
-// of 128-bit weight loads in flight straight into registers and never waits on
-// another wave inside the main loop.
+// Streaming W4A16 kernel for at most 64 activation rows per workgroup (decode
+// and small batch): the weight stream is the roofline, so every wave keeps a
+// ring of 128-bit weight loads in flight straight into registers and never
+// waits on another wave inside the main loop.  A launch covers up to 64 rows,
+// or more where its rows are cut into parts that separate workgroups compute
+// (see the PARTS instance below).
 //
 // Work split (StreamPlan in w4a16_common.hpp): a launch is NT*KG granules of
 // 128 columns x 64 k in column-tile-major order.  A workgroup (4 waves) owns a
