@@ -243,10 +243,17 @@ StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
   sp.gpb = ceil_div(total, cus);
   sp.wpt = 0;
   sp.straddle = !(sp.gpb % KG == 0 || KG % sp.gpb == 0);
-  double best_cost = per_granule * sp.gpb + (sp.straddle ? straddle : 0.0);
+  // the last arrival of a tile fetches its sharers eight at a time: beyond 8
+  // every sharer costs (M = 16, N = 2048, K = 4096: 8 runs per tile 6.1 us,
+  // 16 6.7, 32 10.7; N = 1024, K = 8192: 8 7.9, 16 7.1, 32 8.9)
+  auto sharers = [](int c) {
+    return c <= 8 ? 0.0 : c <= 16 ? 0.1 * (c - 8) : 0.8 + 0.25 * (c - 16);
+  };
+  double best_cost = per_granule * sp.gpb + (sp.straddle ? straddle : 0.0) +
+                     sharers(ceil_div(KG, sp.gpb));
   for (int c = 1; c <= KG && NT * c <= cus; c++) {
     const int g = ceil_div(KG, c);
-    const double cost = per_granule * g;
+    const double cost = per_granule * g + sharers(c);
     if (cost < best_cost + 1e-9) {  // on a tie the one-tile form: its kernel is leaner
       sp.gpb = g;
       sp.wpt = c;
@@ -344,7 +351,11 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   if (m <= kStreamMaxRows && cx.force.row_halves != 1 && cx.counters >= 2) {
     // what the launch gains where make_plan cuts its rows in two
     const StreamSplit split = choose_stream_split(ceil_div(m, 16), n, k, cx.cus);
-    const double gain = split.wpt >= 2 ? halves_gain(m, split.wpt, split.gpb) : 0.0;
+    const int half = 16 * ceil_div(ceil_div(m, 2), 16);
+    const StreamSplit hs = choose_stream_split(half / 16, 2 * n, k, cx.cus);
+    const double gain = split.wpt >= 2 && hs.wpt >= 1 && half < m
+                            ? halves_gain(m, 2 * hs.wpt, ceil_div(k / kGranuleK, 2 * hs.wpt))
+                            : 0.0;
     if (gain > 0.25) stream -= gain;
   }
   int parts, wpt, gpb;
@@ -412,13 +423,18 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
     // the k range once more.  Each half is finished by half as many sharers,
     // with half the rows to sum, store and read back.
     const int half = 16 * ceil_div(ceil_div(rows, 2), 16);
-    const bool can = m <= kStreamMaxRows && half < rows && split.wpt >= 2 && cx.counters >= 2;
-    const bool want = cx.force.row_halves == 2 ||
-                      (cx.force.row_halves == 0 && halves_gain(rows, split.wpt, split.gpb) > 0.25);
-    if (can && want) {
+    // the halves' own split: twice the tiles, half the row blocks
+    const StreamSplit hs = choose_stream_split(half / 16, 2 * n, k, cx.cus);
+    const bool can = m <= kStreamMaxRows && half < rows && split.wpt >= 2 && hs.wpt >= 1 &&
+                     cx.counters >= 2;
+    const bool want =
+        can && (cx.force.row_halves == 2 ||
+                (cx.force.row_halves == 0 &&
+                 halves_gain(rows, 2 * hs.wpt, ceil_div(pl.sp.KG, 2 * hs.wpt)) > 0.25));
+    if (want) {
       pl.row_parts = 2;
       pl.part_rows = half;
-      pl.sp.wpt = split.wpt / 2;
+      pl.sp.wpt = hs.wpt;
       pl.sp.gpb = ceil_div(pl.sp.KG, pl.sp.wpt);
       pl.sp.grid = pl.sp.NT * 2 * pl.sp.wpt;
     }
