@@ -15,6 +15,7 @@ SOURCES = {
     "marlin_host.hip": [],
     "scratch_pool.hip": [],
     "w4a16_stream.hip": [],
+    "w4a16_strip.hip": [],
     "w4a16_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "w4a16_prefill_wide.hip": [],
     "f16_streamk.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],

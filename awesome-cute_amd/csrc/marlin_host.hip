@@ -63,7 +63,7 @@ bool configure_device(int dev) {
   std::lock_guard<std::mutex> lk(g_mu);
   if (g_dev[dev].configured) return true;
   if (configure_stream_kernels() != 0 || configure_prefill_kernels() != 0 ||
-      configure_prefill_wide_kernels() != 0) {
+      configure_prefill_wide_kernels() != 0 || configure_strip_kernels() != 0) {
     set_error(hipGetLastError(), "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
     return false;
   }
@@ -117,7 +117,7 @@ int check_shape(int m, int n, int k, int groupsize, int& thread_k, int& thread_n
 }
 
 struct Plan {
-  int kernel;  // 1 streaming, 2 prefill
+  int kernel;  // 1 streaming, 2 prefill, 3 column strips
   int grid;
   StreamPlan sp;
   int launches;
@@ -126,6 +126,7 @@ struct Plan {
   size_t partial_bytes;  // fp32 partial sums the launch exchanges through scratch (0: none)
   int row_parts;         // streaming, one-tile form: parts the rows are cut into (1: uncut)
   int part_rows;         // rows of a part (the last one has the rest)
+  int strips;            // column-strip kernel: 16-column strips per workgroup (else 0)
 };
 
 constexpr int kStreamMaxRows = 64;
@@ -137,6 +138,7 @@ constexpr int kStreamMaxRows = 64;
 struct Force {
   int kernel = 0, k_slices = 0, tile_rows = 0;
   int row_halves = 0;  // streaming kernel: 0 = by cost, 1 = never cut the rows, 2 = cut them where possible
+  int strips = 0;      // column-strip kernel: 0 = by cost, or 1, 2, 4 strips per workgroup
 };
 thread_local Force t_force;
 
@@ -364,6 +366,23 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   return prefill_cost(m, n, k, cx) <= stream;
 }
 
+// 16-column strips per workgroup of the column-strip kernel
+int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
+  (void)m;
+  (void)k;
+  int cs = cx.force.strips == 1 || cx.force.strips == 2 || cx.force.strips == 4 ? cx.force.strips : 1;
+  while (n % (16 * cs) != 0) cs /= 2;
+  return cs;
+}
+
+bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
+  (void)m;
+  (void)n;
+  (void)k;
+  (void)cx;
+  return false;
+}
+
 Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   Plan pl;
   const int force = cx.force.kernel;
@@ -376,6 +395,15 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   pl.partial_bytes = 0;
   pl.row_parts = 1;
   pl.part_rows = 0;
+  pl.strips = 0;
+  if (m <= 16 && sms <= 0 && (force == 3 || (force == 0 && prefer_strips(m, n, k, cx)))) {
+    pl.kernel = 3;
+    pl.strips = strips_per_workgroup(m, n, k, cx);
+    pl.grid = n / (16 * pl.strips);
+    pl.sp = make_stream_plan(n, k, 1);
+    pl.launches = 1;
+    return pl;
+  }
   if (prefill) {
     // one workgroup per (tile of C, slice of k)
     pl.kernel = 2;
@@ -464,7 +492,24 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
   const int lock_stride = max_par > 16 ? 16 : max_par;
   (void)hipGetLastError();  // an earlier call's error is not this launch's
   int rc = MARLIN_OK;
-  if (pl.kernel == 2) {
+  if (pl.kernel == 3) {
+    GemmArgs a;
+    a.A = A;
+    a.B = B;
+    a.C = C;
+    a.S = s;
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.locks = nullptr;
+    a.lock_stride = 1;
+    a.scratch = nullptr;
+    a.gpb = 0;
+    a.wpt = 0;
+    a.row_parts = 1;
+    a.part_rows = 0;
+    rc = launch_strip(a, groupsize != -1, pl.strips, stream);
+  } else if (pl.kernel == 2) {
     GemmArgs a;
     a.A = A;
     a.B = B;
@@ -669,7 +714,7 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int* out) {
-  for (int i = 0; i < 10; i++) out[i] = 0;
+  for (int i = 0; i < 13; i++) out[i] = 0;
   int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
   if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
   const PlanCtx cx = {cus, kPoolPartialLimit, t_force};
@@ -686,10 +731,14 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[9] = (int)(pl.partial_bytes >> 10);
   out[10] = pl.kernel == 1 ? pl.row_parts : 1;
   out[11] = pl.kernel == 1 ? pl.part_rows : 0;
+  out[12] = pl.strips;
   return rc;
 }
 
-void marlin_amd_force_kernel(int which) { t_force.kernel = which == 1 || which == 2 ? which : 0; }
+void marlin_amd_force_kernel(int which) { t_force.kernel = which >= 1 && which <= 3 ? which : 0; }
+void marlin_amd_force_strips(int strips) {
+  t_force.strips = strips == 1 || strips == 2 || strips == 4 ? strips : 0;
+}
 
 void marlin_amd_force_k_slices(int slices) { t_force.k_slices = slices > 0 ? slices : 0; }
 

@@ -196,6 +196,10 @@ int configure_stream_kernels();
 int configure_prefill_kernels();
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
+// at most 16 rows; a workgroup per `strips` (1, 2 or 4) 16-column strips over
+// the whole k range, nothing exchanged between workgroups (w4a16_strip.hip)
+int configure_strip_kernels();
+int launch_strip(const GemmArgs& a, bool group, int strips, hipStream_t stream);
 // ksplit >= 1 slices of the k range per tile; above 1 the launch needs
 // a.scratch (ksplit * tiles * tile bytes of fp32) and a.locks (one zeroed
 // counter per tile, zero again afterwards)

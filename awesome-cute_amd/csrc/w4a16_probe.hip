@@ -259,7 +259,7 @@ int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, v
   }
   const int cus = info[0];
   // the grid and the work split of a one-row launch of this shape
-  int plan[12];
+  int plan[13];
   const int rc = marlin_amd_plan(1, prob_n, prob_k, -1, -1, -1, -1, cus, plan);
   if (rc != MARLIN_OK) return rc;
   int prev = -1;

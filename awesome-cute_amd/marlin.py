@@ -47,6 +47,8 @@ _lib.marlin_amd_force_row_halves.restype = None
 _lib.marlin_amd_force_row_halves.argtypes = [_I]
 _lib.marlin_amd_force_kernel.restype = None
 _lib.marlin_amd_force_kernel.argtypes = [_I]
+_lib.marlin_amd_force_strips.restype = None
+_lib.marlin_amd_force_strips.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
 _lib.marlin_amd_work_order.argtypes = [_I, _P]
 _lib.marlin_amd_last_error.restype = ctypes.c_char_p
@@ -268,8 +270,15 @@ def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
 
 
 def force_kernel(which):
-    """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel (calling thread only)."""
+    """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel, 3 = column-strip kernel
+    (at most 16 rows; other problems are planned as with 0) -- calling thread only."""
     _lib.marlin_amd_force_kernel(int(which))
+
+
+def force_strips(strips):
+    """16-column strips per workgroup of the column-strip kernel (1, 2 or 4); 0 = choose by
+    cost (calling thread only)."""
+    _lib.marlin_amd_force_strips(int(strips))
 
 
 def force_k_slices(slices):
@@ -298,10 +307,10 @@ def work_order(grid):
 
 def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     """Kernel, grid and stream-K partition marlin_gemm would use."""
-    out = (ctypes.c_int * 12)()
+    out = (ctypes.c_int * 13)()
     rc = _lib.marlin_amd_plan(m, n, k, groupsize, thread_k, thread_n, sms, cus, out)
     keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
-            "k_slices", "tile_rows", "wgs_per_tile", "partial_kib", "row_parts", "part_rows")
+            "k_slices", "tile_rows", "wgs_per_tile", "partial_kib", "row_parts", "part_rows", "strips")
     return rc, dict(zip(keys, out))
 
 

@@ -21,7 +21,8 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
 
 /*
  * How marlin_gemm would run a problem on a device with `cus` compute units:
- * out[0] = kernel (0 = none, 1 = streaming, 2 = prefill), out[1] = workgroups,
+ * out[0] = kernel (0 = none, 1 = streaming, 2 = prefill, 3 = column strips),
+ * out[1] = workgroups,
  * out[2] = granules per workgroup (streaming), out[3] = column tiles,
  * out[4] = granules per column tile, out[5] = number of launches,
  * out[6] = slices of the k range per tile (prefill), out[7] = rows of C per
@@ -31,8 +32,9 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * granules into equal runs of out[2]; out[9] = KiB of partial sums the launch
  * exchanges through the library's scratch (0 = none); out[10] = parts the
  * streaming kernel cuts the rows into (1 = uncut; every part is a problem of
- * its own for out[8] workgroups per column tile), out[11] = rows of a part.
- * `out` holds 12 ints.  Returns the marlin_gemm error code for the shape.
+ * its own for out[8] workgroups per column tile), out[11] = rows of a part;
+ * out[12] = 16-column strips per workgroup of the column-strip kernel (else 0).
+ * `out` holds 13 ints.  Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
                     int thread_n, int sms, int cus, int *out);
@@ -51,11 +53,19 @@ void marlin_amd_work_order(int grid, int *out);
  * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
  * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
  * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is
- * used).  Like the two overrides below it is kept per host thread, so it never
+ * used), 3 = the column-strip kernel (at most 16 rows and no `sms` hint, else
+ * as with 0).  Like the overrides below it is kept per host thread, so it never
  * changes what other threads' calls do.  No reference counterpart; for tests
  * and tools.
  */
 void marlin_amd_force_kernel(int which);
+
+/*
+ * 16-column strips per workgroup of the column-strip kernel, for the calling
+ * thread: 0 = choose by cost (default), or 1, 2, 4 (halved until prob_n is a
+ * multiple of 16 x strips).  No reference counterpart; for tests and tools.
+ */
+void marlin_amd_force_strips(int strips);
 
 /*
  * Slices of the k range per tile of the prefill kernel, for the calling
