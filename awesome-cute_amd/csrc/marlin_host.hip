@@ -133,7 +133,8 @@ constexpr int kStreamMaxRows = 64;
 
 // Overrides of the planner for the calling thread (tests and tools; see
 // marlin_amd_force_*): which kernel (0 = by cost, 1 = streaming in chunks of
-// 64 rows, 2 = prefill), slices of the k range per prefill tile (0 = by cost),
+// 64 rows, 2 = prefill, 3 = column strips, 4 = by cost without the column
+// strips), slices of the k range per prefill tile (0 = by cost),
 // rows of C per prefill workgroup (0 = by cost, 64 or 128).
 struct Force {
   int kernel = 0, k_slices = 0, tile_rows = 0;
@@ -235,6 +236,11 @@ struct StreamSplit {
   int wpt;        // workgroups per column tile, or 0 for the uniform form
   bool straddle;  // workgroups cross tile boundaries
 };
+// The last arrival of a tile fetches its sharers eight at a time: beyond 8
+// every sharer costs (M = 16, N = 2048, K = 4096: 8 runs per tile 6.1 us, 16
+// 6.7, 32 10.7; N = 1024, K = 8192: 8 7.9, 16 7.1, 32 8.9)
+double sharer_cost(int c) { return c <= 8 ? 0.0 : c <= 16 ? 0.1 * (c - 8) : 0.8 + 0.25 * (c - 16); }
+
 StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
   const int NT = n / kTileN;
   const int KG = k / kGranuleK;
@@ -245,12 +251,7 @@ StreamSplit choose_stream_split(int mb, int n, int k, int cus) {
   sp.gpb = ceil_div(total, cus);
   sp.wpt = 0;
   sp.straddle = !(sp.gpb % KG == 0 || KG % sp.gpb == 0);
-  // the last arrival of a tile fetches its sharers eight at a time: beyond 8
-  // every sharer costs (M = 16, N = 2048, K = 4096: 8 runs per tile 6.1 us,
-  // 16 6.7, 32 10.7; N = 1024, K = 8192: 8 7.9, 16 7.1, 32 8.9)
-  auto sharers = [](int c) {
-    return c <= 8 ? 0.0 : c <= 16 ? 0.1 * (c - 8) : 0.8 + 0.25 * (c - 16);
-  };
+  auto sharers = sharer_cost;
   double best_cost = per_granule * sp.gpb + (sp.straddle ? straddle : 0.0) +
                      sharers(ceil_div(KG, sp.gpb));
   for (int c = 1; c <= KG && NT * c <= cus; c++) {
@@ -317,7 +318,8 @@ double stream_cost(int m, int n, int k, int cus) {
     t += full * (tail > 48 ? 1.0 : tail > 32 ? 0.9 : 0.65);
   } else if (tail > 0) {
     const StreamSplit s1 = choose_stream_split(1, n, k, cus);
-    t += 5.1 + 0.16 * s1.gpb + (s1.straddle ? 3.5 : 0.0);
+    t += 5.1 + 0.16 * s1.gpb + (s1.straddle ? 3.5 : 0.0) +
+         sharer_cost(s1.wpt > 0 ? s1.wpt : ceil_div(k / kGranuleK, s1.gpb));
   }
   return t + 1.0 * (ceil_div(m, kStreamMaxRows) - 1);
 }
@@ -366,30 +368,63 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   return prefill_cost(m, n, k, cx) <= stream;
 }
 
-// 16-column strips per workgroup of the column-strip kernel
-int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
-  (void)m;
-  (void)k;
-  int cs = cx.force.strips == 1 || cx.force.strips == 2 || cx.force.strips == 4 ? cx.force.strips : 1;
-  while (n % (16 * cs) != 0) cs /= 2;
-  return cs;
+// Fitted time (us) of the column-strip kernel with `cs` strips per workgroup,
+// at most 16 rows.  A launch costs 2.7 us; a workgroup takes in its 8 cs k
+// bytes of weights and its m rows of activations (from the L2, counted at a
+// quarter) at about 19 GB/s, what its eight waves unpack and multiply;
+// workgroups beyond one per compute unit queue up behind each other, 0.3 us
+// each; all together they draw 4.3 TB/s from memory at most.  Measured
+// (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.4, N = 11008, K = 4096
+// 8.5, N = 1024, K = 8192 6.3, 8192 x 8192 11.3 (two strips 10.8); M = 16:
+// 4096 x 4096 6.3, N = 11008, K = 4096 with four strips 10.9.
+double strip_cost(int m, int n, int k, int cs, int cus) {
+  const int per_cu = ceil_div(n / (16 * cs), cus);
+  const double wg_bytes = 8.0 * cs * k + 0.25 * 2.0 * m * k;
+  const double by_cu = per_cu * wg_bytes / 19e3 + 0.3 * (per_cu - 1);
+  const double by_memory = 0.5 * k * n / 4.3e6;
+  return 2.7 + (by_cu > by_memory ? by_cu : by_memory);
 }
 
+// 16-column strips per workgroup of the column-strip kernel: the cheapest of
+// 1, 2 and 4 that divide n's strips
+int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
+  int best = 0;
+  double best_cost = 0.0;
+  for (int cs = 1; cs <= 4; cs *= 2) {
+    if (n % (16 * cs) != 0) break;
+    if (cx.force.strips != 0 && cx.force.strips != cs && best != 0) continue;
+    const double c = strip_cost(m, n, k, cs, cx.cus);
+    if (best == 0 || cx.force.strips == cs || c < best_cost) {
+      best = cs;
+      best_cost = c;
+      if (cx.force.strips == cs) break;
+    }
+  }
+  return best;
+}
+
+// The column-strip kernel against the streaming kernel for at most 16 rows:
+// the streaming kernel reaches more of the memory's bandwidth (its workgroups
+// share a column tile's k range, so every compute unit has work whatever n
+// is), the strips pay nothing for the exchange between workgroups -- 2 us of a
+// launch that takes 6.  The strips win while the weights are a few MiB per
+// launch (M = 1: 4096 x 4096 4.4 against 6.3 us, N = 11008, K = 4096 8.5
+// against 9.7, 8192 x 8192 10.8 against 10.4 -- there no more) and the rows
+// few (M = 16: 4096 x 4096 6.3 against 6.6, N = 11008 10.9 against 9.9).
 bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
-  (void)m;
-  (void)n;
-  (void)k;
-  (void)cx;
-  return false;
+  const int cs = strips_per_workgroup(m, n, k, cx);
+  return strip_cost(m, n, k, cs, cx.cus) < stream_cost(m, n, k, cx.cus);
 }
 
 Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   Plan pl;
-  const int force = cx.force.kernel;
+  // (the column-strip kernel does at most 16 rows and takes no hint: forced
+  // onto anything else it leaves the choice to the costs)
+  const int force = cx.force.kernel == 3 && (m > 16 || sms > 0) ? 0 : cx.force.kernel;
   // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
   // whenever m > 16, by the shape contract)
-  const bool prefill =
-      n % 256 == 0 && (force == 2 || (force == 0 && prefer_prefill(m, n, k, cx)));
+  const bool by_cost = force == 0 || force == 4;
+  const bool prefill = n % 256 == 0 && (force == 2 || (by_cost && prefer_prefill(m, n, k, cx)));
   pl.ksplit = 1;
   pl.tile_rows = 0;
   pl.partial_bytes = 0;
@@ -735,7 +770,7 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   return rc;
 }
 
-void marlin_amd_force_kernel(int which) { t_force.kernel = which >= 1 && which <= 3 ? which : 0; }
+void marlin_amd_force_kernel(int which) { t_force.kernel = which >= 1 && which <= 4 ? which : 0; }
 void marlin_amd_force_strips(int strips) {
   t_force.strips = strips == 1 || strips == 2 || strips == 4 ? strips : 0;
 }

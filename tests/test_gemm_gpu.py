@@ -30,6 +30,18 @@ def env():
     return torch, marlin
 
 
+@pytest.fixture
+def no_strips(env):
+    """Up to 16 rows through the streaming kernel, as larger launches go: for
+    the tests of what workgroups exchange (partial sums, tickets, scratch),
+    which the column-strip kernel, the planner's choice for few rows over small
+    weights, does not have."""
+    torch, marlin = env
+    marlin.force_kernel(4)
+    yield
+    marlin.force_kernel(0)
+
+
 def gpu_gemm(env, A, B, sp, N, thread_k=-1, thread_n=-1, sms=-1, max_par=16, C_fill=None):
     torch, marlin = env
     dev = torch.device("cuda:0")
@@ -146,14 +158,14 @@ def test_partition_sweep(env, sms, groupsize):
     check(env, 48, 768, 2048, groupsize, seed=sms + 1, sms=sms)
 
 
-def test_deterministic(env):
+def test_deterministic(env, no_strips):
     A, q, s, B, sp = O.make_problem(16, 4096, 4096, 128, seed=9)
     c1 = gpu_gemm(env, A, B, sp, 4096)
     c2 = gpu_gemm(env, A, B, sp, 4096)
     assert np.array_equal(c1.view(np.uint16), c2.view(np.uint16))
 
 
-def test_partition_does_not_change_the_bits(env):
+def test_partition_does_not_change_the_bits(env, no_strips):
     """Partial sums are added in workgroup order by whoever arrives last, so a
     given partition always gives the same bits; different partitions differ
     only by fp32 reassociation (inside the tolerance)."""
@@ -172,7 +184,7 @@ def test_workspace_stride_follows_max_par(env, max_par):
     check(env, 33, 512, 1024, -1, seed=max_par + 1, max_par=max_par, sms=24)
 
 
-def test_back_to_back_launches_share_scratch(env):
+def test_back_to_back_launches_share_scratch(env, no_strips):
     """Launches on one stream reuse the partial-sum slots: different inputs of
     one shape, and then another shape, must not see each other's partial sums."""
     torch, marlin = env
@@ -196,7 +208,7 @@ def test_back_to_back_launches_share_scratch(env):
         assert not ws.any().item()
 
 
-def test_two_streams_run_side_by_side(env):
+def test_two_streams_run_side_by_side(env, no_strips):
     """GEMMs on two streams at the same time: each stream has its own partial-sum
     scratch, so neither sees the other's.  Shared column tiles (streaming kernel)
     and k slices (prefill kernel) on both; every result equals the one the same
@@ -235,7 +247,7 @@ def test_two_streams_run_side_by_side(env):
             assert not ws.any().item()
 
 
-def test_kernels_of_other_streams_beside_do_not_change_the_result(env):
+def test_kernels_of_other_streams_beside_do_not_change_the_result(env, no_strips):
     """A launch gives the same bits whatever else runs on the GPU: kernels of another
     stream that keep LDS and memory busy stretch every latency inside the GEMM, which
     must not matter (shared column tiles of the streaming kernel with 1, 16 and 64 rows,
@@ -271,7 +283,7 @@ def test_kernels_of_other_streams_beside_do_not_change_the_result(env):
         assert all(torch.equal(c, alone) for c in outs), (m, n, k)
 
 
-def test_two_host_threads_two_streams(env):
+def test_two_host_threads_two_streams(env, no_strips):
     """Two host threads, each with a stream of its own, call the library at the same time
     (ctypes releases the interpreter lock during a call): the per-device state behind the
     C ABI is locked, and both get the results a single thread gets."""
@@ -288,6 +300,7 @@ def test_two_host_threads_two_streams(env):
 
     def worker():
         try:
+            marlin.force_kernel(4)  # kept per host thread
             st = torch.cuda.Stream()
             with torch.cuda.stream(st):
                 ws = torch.zeros(2048 // 128 * 16, dtype=torch.int, device=dev)
@@ -492,6 +505,111 @@ def test_more_than_64_rows_in_one_streaming_launch(env, m, groupsize):
     finally:
         marlin.force_kernel(0)
         marlin.force_row_halves(0)
+
+
+STRIP_SHAPES = [
+    # (m, n, k, groupsize): rows for every count of staged rows (2, 4, 8, 16), one chunk
+    # and a ragged last one, runs of more chunks than the ring holds, both scale modes
+    (1, 256, 256, 128), (2, 128, 128, -1), (3, 512, 2304, -1), (4, 2048, 1408, 128),
+    (5, 768, 512, 128), (8, 640, 13824, 128), (9, 1280, 1152, 128), (13, 896, 384, -1),
+    (16, 256, 4096, 128), (16, 128, 128, -1), (7, 384, 640, -1), (16, 2048, 128 * 37, 128),
+    (11, 1152, 64 * 2 * 51, -1), (1, 1024, 8192, -1), (16, 4096, 4096, -1), (1, 11008, 4096, 128),
+]
+
+
+@pytest.mark.parametrize("strips", [1, 2, 4])
+@pytest.mark.parametrize("m,n,k,g", STRIP_SHAPES)
+def test_column_strip_kernel(env, strips, m, n, k, g):
+    """The kernel for at most 16 rows whose workgroups own 16, 32 or 64 columns
+    over the whole k range and exchange nothing: every strip width on every
+    shape, C overwritten everywhere (it starts at 9)."""
+    torch, marlin = env
+    marlin.force_kernel(3)
+    marlin.force_strips(strips)
+    try:
+        rc, p = marlin.plan(m, n, k, g)
+        assert (rc, p["kernel"], p["strips"], p["grid"]) == (0, 3, strips, n // (16 * strips))
+        A, q, s, B, sp = O.make_problem(m, n, k, g, seed=m + n + k)
+        C = gpu_gemm(env, A, B, sp, n, C_fill=9.0)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_strips(0)
+    r = O.compare(C, O.gemm(A, B, sp, n, -1 if g == k else g))
+    assert r.max_abs_err <= TOL * r.max_abs_ref, (r.max_abs_err, r.max_abs_ref)
+    assert r.rel_mean_abs_err <= REL_MEAN_TOL, r.rel_mean_abs_err
+
+
+@pytest.mark.parametrize("strips", [1, 2, 4])
+@pytest.mark.parametrize("groupsize", [128, -1])
+def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsize):
+    """One-hot rows through the column strips return the dequantised weights bit
+    for bit: every k of a 1024-deep weight (16 rows at a time: all staged-row
+    counts' widest instance), then single rows and short batches (the narrower
+    instances), for every strip width and both scale modes."""
+    torch, marlin = env
+    N, K = 256, 1024
+    _, q, s, B, sp = O.make_problem(1, N, K, groupsize, seed=13)
+    W = O.dequant(B, sp, K, N, groupsize)
+    if groupsize == -1:
+        W = W * O.unpack_scales(sp, False)  # fp16(q-8) * s, one rounding
+    marlin.force_kernel(3)
+    marlin.force_strips(strips)
+    try:
+        for base in range(0, K, 16):
+            A = np.zeros((16, K), np.float16)
+            A[np.arange(16), base + np.arange(16)] = 1.0
+            C = gpu_gemm(env, A, B, sp, N)
+            assert np.array_equal(C.view(np.uint16), W[base:base + 16].view(np.uint16)), base
+        for rows in ([0], [1023], [5, 700], [17, 130, 511], [3, 64, 65, 1000], list(range(2, 1024, 171))[:6]):
+            A = np.zeros((len(rows), K), np.float16)
+            for i, r in enumerate(rows):
+                A[i, r] = 1.0
+            C = gpu_gemm(env, A, B, sp, N)
+            assert np.array_equal(C.view(np.uint16), W[rows].view(np.uint16)), rows
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_strips(0)
+
+
+@pytest.mark.parametrize("strips", [1, 2, 4])
+def test_column_strip_kernel_closed_forms(env, strips):
+    """Zero point everywhere gives exact zeros; small integers times unit scales
+    give exact integers (every product and every partial sum is exact in fp32)."""
+    torch, marlin = env
+    M, N, K = 16, 256, 768
+    rng = np.random.default_rng(50 + strips)
+    marlin.force_kernel(3)
+    marlin.force_strips(strips)
+    try:
+        A = rng.standard_normal((M, K)).astype(np.float16)
+        s = rng.uniform(0.001, 0.02, (K // 128, N)).astype(np.float16)
+        q = np.full((K, N), 8, np.uint8)
+        C = gpu_gemm(env, A, O.pack_weights(q), O.pack_scales(s, True), N, C_fill=7.0)
+        assert not C.view(np.uint16).any()
+        Ai = rng.integers(-3, 4, (M, K)).astype(np.float16)
+        q = rng.integers(0, 16, (K, N), dtype=np.uint8)
+        ones = np.ones((K // 128, N), np.float16)
+        C = gpu_gemm(env, Ai, O.pack_weights(q), O.pack_scales(ones, True), N)
+        want = Ai.astype(np.int64) @ (q.astype(np.int64) - 8)
+        assert np.abs(want).max() < 2048
+        assert np.array_equal(C.astype(np.int64), want)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_strips(0)
+
+
+def test_few_rows_through_either_kernel_agree_with_the_oracle(env):
+    """The shapes the planner gives to the column strips, through the streaming
+    kernel as well: both inside the tolerance, on the same inputs."""
+    torch, marlin = env
+    for (m, n, k, g) in [(1, 4096, 4096, 128), (8, 2048, 2048, -1), (16, 1280, 1152, 128)]:
+        assert marlin.plan(m, n, k, g)[1]["kernel"] == 3
+        for which in (0, 4):
+            marlin.force_kernel(which)
+            try:
+                check(env, m, n, k, g, seed=m + k)
+            finally:
+                marlin.force_kernel(0)
 
 
 @pytest.mark.parametrize("tag,groupsize", [("g128", 128), ("chan", -1)])
@@ -706,7 +824,7 @@ def test_llama_larger_shapes(env, model, layer):
             assert r.rel_mean_abs_err <= REL_MEAN_TOL
 
 
-def test_scratch_is_sized_by_the_plan_and_can_be_released(env):
+def test_scratch_is_sized_by_the_plan_and_can_be_released(env, no_strips):
     """Partial-sum scratch: nothing for a launch that exchanges nothing, whole MiB
     sized by the plan per (device, stream) otherwise, shared with the dense
     GEMM, grown on demand, freed by release(); a first call under graph capture
@@ -814,7 +932,7 @@ def test_random_shapes_kernels_and_knobs(env, seed):
         K = 128 * int(rng.integers(1, 40))
         if K == 128 and g == 128:
             K = 256
-        forced = int(rng.choice([0, 0, 1, 2])) if N % 256 == 0 else 0
+        forced = int(rng.choice([0, 0, 1, 2, 3, 4])) if N % 256 == 0 else int(rng.choice([0, 3, 4]))
         rows = int(rng.choice([0, 64, 128]))
         sms = int(rng.choice([-1, -1, -1, 7, 64, 100, 256, 300, 1000]))
         assert marlin.check(M, N, K, g) == 0
@@ -959,14 +1077,23 @@ def test_profiling_row(env, groupsize):
     assert float(row['max_rel_err']) <= TOL
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (48, 1024, 4096), (200, 2048, 2048)])
-def test_graph_replays_match_eager(env, m, n, k):
-    """A captured launch (streaming kernel with shared tiles, LDS-ring variant, prefill
-    kernel with k slices) replayed several times, with eager launches and
+@pytest.mark.parametrize("m,n,k,which", [(1, 4096, 4096, 4), (1, 4096, 4096, 3), (48, 1024, 4096, 0),
+                                         (200, 2048, 2048, 0)])
+def test_graph_replays_match_eager(env, m, n, k, which):
+    """A captured launch (streaming kernel with shared tiles, column strips, LDS-ring
+    variant, prefill kernel with k slices) replayed several times, with eager launches and
     synchronisations in between, gives the eager result every time and leaves the
     workspace zero: the counters are reset by the kernels, nothing is a memset."""
     torch, marlin = env
     dev = torch.device("cuda:0")
+    marlin.force_kernel(which)
+    try:
+        _graph_replays(torch, marlin, dev, m, n, k)
+    finally:
+        marlin.force_kernel(0)
+
+
+def _graph_replays(torch, marlin, dev, m, n, k):
     A, q, s, B, sp = O.make_problem(m, n, k, 128, 41)
     A2, q2, s2, B2, sp2 = O.make_problem(16, 512, 1024, 128, 42)
     d = [torch.from_numpy(x).to(dev) for x in (A, B, sp, A2, B2, sp2)]

@@ -191,7 +191,11 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
     """Without an `sms` hint the planner picks splits whose workgroups never
     straddle a column-tile boundary (one exchange per workgroup at most) and
     never launches more workgroups than CUs."""
-    rc, plan = marlin.plan(m, n, k, -1, -1, -1, -1, 256)
+    marlin.force_kernel(1)  # the streaming kernel's plan, also where column strips would be cheaper
+    try:
+        rc, plan = marlin.plan(m, n, k, -1, -1, -1, -1, 256)
+    finally:
+        marlin.force_kernel(0)
     assert rc == 0 and plan["kernel"] == 1 and plan["grid"] <= 256
     owner = _partition(plan)
     KG = plan["granules_per_tile"]
@@ -207,14 +211,17 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
 
 
 def test_kernel_choice_by_cost(marlin):
-    """Few rows go through the streaming kernel, many through the prefill
+    """Up to 16 rows over a few MiB of weights go through the column-strip
+    kernel, few rows otherwise through the streaming kernel, many through the prefill
     kernel, whose k range is cut into slices (the cheapest count, at most eight)
     while tiles alone would leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
     so do more rows while twice as many tiles save k slices; up to a few hundred
     rows over small weights stream in one launch with the rows cut into parts of
     32.  The knobs override the choice."""
     for m, n, k, kernel, slices, rows in [
-            (1, 4096, 4096, 1, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
+            (1, 4096, 4096, 3, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
+            (1, 11008, 4096, 3, 1, 0), (1, 28672, 8192, 1, 1, 0), (17, 4096, 4096, 1, 1, 0),
+            (8, 2048, 2048, 3, 1, 0), (16, 8192, 8192, 1, 1, 0),
             (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 1, 1, 0),
             (128, 4096, 4096, 1, 1, 0), (512, 4096, 4096, 2, 2, 64),
             (128, 8192, 8192, 2, 4, 64), (640, 4096, 11008, 2, 3, 128),
@@ -231,8 +238,29 @@ def test_kernel_choice_by_cost(marlin):
     assert p["grid"] == 32 * 4 * 2
     rc, p = marlin.plan(64, 4096, 4096, 128)
     assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 2, 32, 4)
-    rc, p = marlin.plan(16, 4096, 4096, 128)
-    assert (p["row_parts"], p["wgs_per_tile"]) == (1, 8)
+    rc, p = marlin.plan(16, 4096, 11008, 128)
+    assert (p["kernel"], p["row_parts"], p["wgs_per_tile"], p["strips"]) == (1, 1, 8, 0)
+    # column strips: a workgroup per 16, 32 or 64 columns, nothing exchanged, one launch
+    rc, p = marlin.plan(1, 4096, 4096, 128)
+    assert (p["kernel"], p["strips"], p["grid"], p["launches"], p["partial_kib"]) == (3, 1, 256, 1, 0)
+    rc, p = marlin.plan(1, 8192, 1024, 128)
+    assert (p["kernel"], p["strips"], p["grid"]) == (3, 2, 256)
+    assert marlin.plan(1, 4096, 4096, 128, sms=64)[1]["kernel"] == 1  # a hint asks for the streaming split
+    try:
+        marlin.force_kernel(3)
+        for strips in (1, 2, 4):
+            marlin.force_strips(strips)
+            rc, p = marlin.plan(16, 28672, 8192, 128)
+            assert (p["kernel"], p["strips"], p["grid"]) == (3, strips, 28672 // (16 * strips))
+        marlin.force_strips(4)
+        rc, p = marlin.plan(16, 128 * 3, 512, 128, 128, 128)  # 24 strips
+        assert (p["kernel"], p["strips"]) == (3, 4) and p["grid"] == 6
+        marlin.force_strips(0)
+        assert marlin.plan(17, 4096, 4096, 128)[1]["kernel"] == 1  # more than 16 rows: as by cost
+        assert marlin.plan(2048, 4096, 4096, 128)[1]["kernel"] == 2
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_strips(0)
     try:
         marlin.force_kernel(1)
         rc, p = marlin.plan(2048, 4096, 4096, 128)
@@ -259,7 +287,7 @@ def test_kernel_choice_by_cost(marlin):
 
 
 def test_plan_picks_kernels(marlin):
-    assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 1
+    assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 3
     assert marlin.plan(32, 28672, 8192, 128)[1]["kernel"] == 1
     rc, p = marlin.plan(2048, 4096, 4096, 128)
     assert rc == 0 and p["kernel"] == 2 and p["grid"] == 16 * 16
@@ -381,12 +409,18 @@ def test_scratch_accounting_and_plan_sizes_without_gpu(marlin):
     slice for the prefill kernel, nothing otherwise."""
     assert marlin.scratch_bytes() == (0, 0)
     assert marlin.release() == 0
-    rc, p = marlin.plan(1, 4096, 4096, 128)
+    rc, p = marlin.plan(1, 4096, 4096, 128)  # column strips: nothing exchanged
+    assert rc == 0 and p["kernel"] == 3 and p["partial_kib"] == 0
+    rc, p = marlin.plan(16, 4096, 11008, 128)
     assert rc == 0 and p["wgs_per_tile"] == 8 and p["grid"] == 256 and p["partial_kib"] == 2 * 256 * 8
     rc, p = marlin.plan(64, 4096, 4096, 128, sms=100)  # forced uniform runs, four row blocks
     assert p["kernel"] == 1 and p["wgs_per_tile"] == 0
     assert p["partial_kib"] == 2 * p["grid"] * 4 * 8
-    rc, p = marlin.plan(16, 256 * 128, 1024, 128, 128, 128)  # one whole tile per workgroup
+    marlin.force_kernel(1)
+    try:
+        rc, p = marlin.plan(16, 256 * 128, 1024, 128, 128, 128)  # one whole tile per workgroup
+    finally:
+        marlin.force_kernel(0)
     assert p["kernel"] == 1 and p["partial_kib"] == 0
     rc, p = marlin.plan(2048, 4096, 4096, 128)
     assert p["kernel"] == 2 and p["k_slices"] == 1 and p["partial_kib"] == 0

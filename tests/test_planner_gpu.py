@@ -1,8 +1,10 @@
-"""Guard of the host's kernel choice (marlin_host.hip: make_plan): on a dozen
-shapes between the decode and the prefill regime, the planned launch must not
+"""Guard of the host's kernel choice (marlin_host.hip: make_plan): on two
+dozen shapes from the decode to the prefill regime, the planned launch must not
 be more than 10 % slower than the best of the forced alternatives -- the
 streaming kernel, the prefill kernel on 64-row tiles and on 128-row tiles, each
-with the slice count its cost model picks.  The planner is a fitted cost model;
+with the slice count its cost model picks, and for at most 16 rows the
+column-strip kernel with 1, 2 and 4 strips per workgroup instead of the prefill
+kernel.  The planner is a fitted cost model;
 this test is what fails when a kernel change shifts the costs under it.  (The
 dispatch rules it replaces: reference marlin_cute_kernel.cu:39-49.)
 """
@@ -18,6 +20,9 @@ sys.path.insert(0, os.path.join(ROOT, "awesome-cute_amd"))
 
 SHAPES = [(m, n, k) for (n, k) in [(4096, 4096), (4096, 11008), (8192, 8192)]
           for m in (48, 64, 128, 512)]
+SHAPES += [(m, n, k) for (n, k) in [(4096, 4096), (11008, 4096), (4096, 11008), (2048, 2048),
+                                    (8192, 8192), (1024, 8192)]
+           for m in (1, 16)]
 SLACK = 1.10
 
 
@@ -67,13 +72,20 @@ def _measure(torch, marlin, m, n, k):
         times["planned"] = _us_per_call(torch, call, 40)
         marlin.force_kernel(1)
         times["streaming"] = _us_per_call(torch, call, 40)
-        for rows in (64, 128):
-            marlin.force_kernel(2)
-            marlin.force_tile_rows(rows)
-            times[f"prefill, {rows}-row tiles"] = _us_per_call(torch, call, 40)
+        if m <= 16:
+            for strips in (1, 2, 4):
+                marlin.force_kernel(3)
+                marlin.force_strips(strips)
+                times[f"column strips, {strips} per workgroup"] = _us_per_call(torch, call, 40)
+        else:
+            for rows in (64, 128):
+                marlin.force_kernel(2)
+                marlin.force_tile_rows(rows)
+                times[f"prefill, {rows}-row tiles"] = _us_per_call(torch, call, 40)
     finally:
         marlin.force_kernel(0)
         marlin.force_tile_rows(0)
+        marlin.force_strips(0)
     torch.cuda.synchronize()
     assert not ws.any().item()
     return times

@@ -30,6 +30,17 @@ def env():
     return torch, marlin
 
 
+@pytest.fixture(autouse=True)
+def no_strips(env):
+    """This file is about the scratch: few rows go through the streaming
+    kernel, which exchanges partial sums, not through the column strips, which
+    the planner would pick for them and which use no scratch at all."""
+    torch, marlin = env
+    marlin.force_kernel(4)
+    yield
+    marlin.force_kernel(0)
+
+
 def both(env, M, N, K, g, seed, sms=-1):
     """marlin_gemm_static and marlin_gemm on the same device buffers."""
     torch, marlin = env
@@ -85,6 +96,18 @@ def test_static_matches_pool_entry(env, M, N, K, g, sms):
     assert r.max_abs_err <= TOL * r.max_abs_ref
 
 
+def test_static_entry_through_column_strips(env):
+    """The planner's own choice for few rows over small weights: no scratch on
+    either entry, the same bits."""
+    torch, marlin = env
+    marlin.force_kernel(0)
+    assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 3
+    (A, B, sp), c_static, c_pool = both(env, 1, 4096, 4096, 128, seed=77)
+    assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
+    r = O.compare(c_static, O.gemm(A, B, sp, 4096, 128))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
+
+
 def test_rejects_what_does_not_fit(env):
     """Only an explicit grid hint above the device's compute units with more than
     16 rows needs more than the fixed 32 MiB: a clear error, nothing launched."""
@@ -100,7 +123,7 @@ def test_rejects_what_does_not_fit(env):
     try:
         rc = marlin.gemm_raw("marlin_gemm_static", dA, dB, dC, ds, ws, 128, sms=1000)
     finally:
-        marlin.force_kernel(0)
+        marlin.force_kernel(4)
     assert rc == 3 and "fixed scratch holds 33554432" in marlin.last_error()
     torch.cuda.synchronize()
     assert (dC == 3.0).all().item() and not ws.any().item()
