@@ -9,7 +9,10 @@
 // does for the same plan -- same work split, same workgroup-to-XCD order, same
 // 128-bit streaming buffer loads of 1 KiB per wave instruction, four rows per
 // granule -- keeps up to kProbeDepth granules in flight per wave, and throws
-// the data away.  probe_empty_kernel does nothing at all.  probe_mfma_kernel is
+// the data away; probe_read_strips_kernel does the same for the column-strip
+// kernel's split (a workgroup of eight waves per 16, 32 or 64 columns over the
+// whole k range, eight rows of a strip per wave instruction).
+// probe_empty_kernel does nothing at all.  probe_mfma_kernel is
 // a loop of nothing but v_mfma_f32_16x16x32_f16 on pseudo-random operands, two
 // waves per SIMD and 32 independent accumulators per wave: what the matrix
 // pipes of this board sustain when nothing competes with them.
@@ -26,7 +29,7 @@ constexpr int kProbeDepth = 4;
 constexpr int kProbeOob = (int)0x80000000;
 }  // namespace
 
-__global__ __launch_bounds__(256) void probe_empty_kernel() {}
+__global__ __launch_bounds__(512) void probe_empty_kernel() {}
 
 __global__ __launch_bounds__(256) void probe_read_kernel(GemmArgs p, int* sink) {
   const int tid = threadIdx.x;
@@ -73,6 +76,46 @@ __global__ __launch_bounds__(256) void probe_read_kernel(GemmArgs p, int* sink) 
     }
   }
   // uniform packed nibbles never OR to this pattern: nothing is written
+  if ((acc[0] & acc[1] & acc[2] & acc[3]) == 0x12345678 && sink) sink[0] = 1;
+}
+
+template <int CS>
+__global__ __launch_bounds__(512) void probe_read_strips_kernel(GemmArgs p, int* sink) {
+  constexpr int kRows = 16 / CS;  // rows of B per chunk: two loads of 1 KiB per wave
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int wid = xcd_work_index((int)blockIdx.x, (int)gridDim.x);
+  const int strip0 = wid * CS;
+  const int n_chunks = ceil_div(p.K, 16 * kRows);
+  const int c0 = (wave * n_chunks) / 8, c1 = ((wave + 1) * n_chunks) / 8;
+  const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void*>(p.B), 0, (int)((unsigned)p.K * (unsigned)(p.N / 2)), 0x00020000);
+  const int b_row = p.N * 8;
+  int b_lane[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int idx = 64 * i + lane;
+    b_lane[i] = (idx / (8 * CS)) * b_row + 128 * (strip0 + (idx / 8) % CS) + 16 * (idx % 8);
+  }
+  i4 acc = {0, 0, 0, 0};
+  i4 buf[kProbeDepth][2];
+  auto issue = [&](int slot, int c) {
+    const int inv = c < c1 ? 0 : kProbeOob;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      buf[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
+          rB, (b_lane[i] + c * kRows * b_row) | inv, 0, 2);
+  };
+#pragma unroll
+  for (int d = 0; d < kProbeDepth; d++) issue(d, c0 + d);
+  for (int c = c0; c < c1; c += kProbeDepth) {
+#pragma unroll
+    for (int d = 0; d < kProbeDepth; d++) {
+      acc |= buf[d][0] | buf[d][1];
+      issue(d, c + d + kProbeDepth);
+    }
+  }
   if ((acc[0] & acc[1] & acc[2] & acc[3]) == 0x12345678 && sink) sink[0] = 1;
 }
 
@@ -247,20 +290,25 @@ bool run_and_fetch(int n, float* host_out, F fn) {
 
 extern "C" {
 
-int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, void* stream_) {
+int marlin_amd_probe(int kind, const void* B, int prob_m, int prob_n, int prob_k, int dev,
+                     void* stream_) {
   using namespace w4a16;
   hipStream_t stream = (hipStream_t)stream_;
   g_probe_error[0] = 0;
-  if (prob_n <= 0 || prob_k <= 0 || dev < 0 || kind < 0 || kind > 2) return MARLIN_ERR_PROB_SHAPE;
+  if (prob_m <= 0 || prob_n <= 0 || prob_k <= 0 || dev < 0 || kind < 0 || kind > 2)
+    return MARLIN_ERR_PROB_SHAPE;
   int info[5] = {0, 0, 0, 0, 0};
   if (marlin_amd_device_info(dev, info) != MARLIN_OK || info[0] <= 0) {
     snprintf(g_probe_error, sizeof(g_probe_error), "device %d: %s", dev, marlin_amd_last_error());
     return MARLIN_ERR_RUNTIME;
   }
   const int cus = info[0];
-  // the grid and the work split of a one-row launch of this shape
+  // the grid and the work split of a launch of this shape with prob_m rows; where
+  // that is the prefill kernel's, of a launch with 16 rows
   int plan[13];
-  const int rc = marlin_amd_plan(1, prob_n, prob_k, -1, -1, -1, -1, cus, plan);
+  int rc = marlin_amd_plan(prob_m, prob_n, prob_k, -1, -1, -1, -1, cus, plan);
+  if (rc == MARLIN_OK && plan[0] == 2)
+    rc = marlin_amd_plan(16, prob_n, prob_k, -1, -1, -1, -1, cus, plan);
   if (rc != MARLIN_OK) return rc;
   int prev = -1;
   hipError_t e = hipGetDevice(&prev);
@@ -271,8 +319,21 @@ int marlin_amd_probe(int kind, const void* B, int prob_n, int prob_k, int dev, v
   }
   (void)hipGetLastError();
   const int grid = plan[1];
+  const int strips = plan[0] == 3 ? plan[12] : 0;
   if (kind == 0) {
-    hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(256), 0, stream);
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(grid), dim3(strips ? 512 : 256), 0, stream);
+  } else if (kind == 1 && strips) {
+    GemmArgs a = {};
+    a.B = B;
+    a.M = 1;
+    a.N = prob_n;
+    a.K = prob_k;
+    if (strips == 1)
+      hipLaunchKernelGGL(probe_read_strips_kernel<1>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
+    else if (strips == 2)
+      hipLaunchKernelGGL(probe_read_strips_kernel<2>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
+    else
+      hipLaunchKernelGGL(probe_read_strips_kernel<4>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
   } else if (kind == 1) {
     GemmArgs a = {};
     a.B = B;

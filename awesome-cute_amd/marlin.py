@@ -358,7 +358,7 @@ def _probes():
             raise RuntimeError(f"{path} is missing: build it (python awesome-cute_amd/build.py)")
         lib = ctypes.CDLL(path)
         lib.marlin_amd_probe.restype = _I
-        lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _P]
+        lib.marlin_amd_probe.argtypes = [_I, _P, _I, _I, _I, _I, _P]
         lib.marlin_amd_probe_issue.restype = _I
         lib.marlin_amd_probe_issue.argtypes = [_I, _I, _I, _I, _I, _P]
         lib.marlin_amd_probe_pull.restype = _I
@@ -374,12 +374,12 @@ def _probe_check(rc, what):
                            f"{_probes().marlin_amd_probe_last_error().decode()}")
 
 
-def probe(kind, B, n, k):
+def probe(kind, B, n, k, m=1):
     """Measurement probe on the current stream: kind 0 = empty launch, 1 = plain read of the
-    packed weights B with the streaming kernel's work split, 2 = a loop of nothing but MFMAs
-    (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe)."""
+    packed weights B with the work split of the kernel planned for m rows of this shape, 2 = a
+    loop of nothing but MFMAs (n*k/8192 per wave, 8 waves per compute unit) (marlin_amd_probe)."""
     dev = B.get_device()
-    _probe_check(_probes().marlin_amd_probe(kind, B.data_ptr(), n, k, dev, _raw_stream(dev)),
+    _probe_check(_probes().marlin_amd_probe(kind, B.data_ptr(), m, n, k, dev, _raw_stream(dev)),
                  "marlin_amd_probe")
 
 

@@ -65,8 +65,8 @@ M_SWEEP = ["m32", "m64", "m128", "m256", "m512", "m1024"]
 # it was measured on (kernel, grid): when the library plans the shape otherwise
 # the figure is stale and is reported as null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode": (("stream", 256), int((4760.5 * 2.0 + 273.0) * 1024)),          # 10.0 MB, 1.16 x algorithmic
-    "batch16": (("stream", 256), int((5688.5 * 2.0 + 2185.0) * 1024)),        # 13.9 MB, 1.56 x (2 MiB of partial sums)
+    "decode": (("strips", 256), int((4297.0 * 2.0 + 8.0) * 1024)),            # 8.81 MB, 1.02 x algorithmic
+    "batch16": (("strips", 256), int((4782.5 * 2.0 + 128.0) * 1024)),         # 9.93 MB, 1.11 x (the rows read by every workgroup)
     "prefill": (("prefill", 256), int((33941.5 * 2.0 + 16389.5) * 1024)),     # 86.3 MB, 2.04 x (A and B read by 16 tiles each)
     "mlp_up": (("stream", 172), int((12296.0 * 2.0 + 1728.1) * 1024)),        # 27.0 MB, 1.14 x
     "mlp_down": (("stream", 256), int((13714.5 * 2.0 + 2185.0) * 1024)),      # 30.3 MB, 1.28 x
@@ -202,15 +202,16 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=Fal
     floor = None
     if with_floor and bound == "hbm":
         # what the launch alone and the weight stream alone cost, measured the same way
-        e_ms, _ = graph_ms(torch, side, lambda i: marlin.probe(0, dBs[0], N, K), steps, 1)
-        r_ms, r_spread = graph_ms(torch, side, lambda i: marlin.probe(1, dBs[i % nbuf], N, K),
+        e_ms, _ = graph_ms(torch, side, lambda i: marlin.probe(0, dBs[0], N, K, M), steps, 1)
+        r_ms, r_spread = graph_ms(torch, side, lambda i: marlin.probe(1, dBs[i % nbuf], N, K, M),
                                   steps, nbuf)
         floor = {"empty_kernel_us": e_ms * 1e3, "read_kernel_us": r_ms * 1e3,
                  "read_kernel_spread_us": [x * 1e3 for x in r_spread[:2]],
                  "read_GBps": weight_bytes / (r_ms * 1e-3) / 1e9,
-                 "what": "same grid and work split as a one-row launch of this shape; read kernel = "
-                         "the packed weights through the streaming kernel's 128-bit loads, no "
-                         "arithmetic, nothing written; same buffer rotation and graph timing"}
+                 "what": "same grid and work split as the kernel planned for this launch (for 16 "
+                         "rows where that is the prefill kernel); read kernel = the packed weights "
+                         "through that kernel's 128-bit loads, no arithmetic, nothing written; same "
+                         "buffer rotation and graph timing"}
     elif with_floor:
         # what the matrix pipes sustain on the same count of multiply-adds with
         # nothing beside them (one workgroup of 8 waves per CU, N*K/8192 MFMAs
@@ -238,7 +239,7 @@ def time_shape(torch, marlin, O, name, steps, warmup, check=True, with_floor=Fal
         "cache_resident_us_per_launch": None if resident_ms is None else resident_ms * 1e3,
     }
     rc, plan = marlin.plan(M, N, K, g, -1, -1, -1, marlin.device_info(0)["compute_units"])
-    kernel = {1: "stream", 2: "prefill"}.get(plan["kernel"])
+    kernel = {1: "stream", 2: "prefill", 3: "strips"}.get(plan["kernel"])
     res["plan"] = {"kernel": kernel, "grid": plan["grid"], "k_slices": plan["k_slices"],
                    "tile_rows": plan["tile_rows"]}
     measured_on, traffic = MEASURED_TRAFFIC_BYTES.get(name, (None, None))
@@ -356,6 +357,11 @@ def main():
                     help="headline (decode, then the other benchmark shapes) or one of: " +
                          ", ".join(SHAPES))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernel", type=int, default=0,
+                    help="0 (default) = the library's own choice of kernel; 1 streaming, 2 prefill, "
+                         "3 column strips, 4 = by cost without the column strips "
+                         "(marlin_amd_force_kernel): to time or profile an alternative; such a "
+                         "run is not the benchmark")
     ap.add_argument("--extras", action="store_true",
                     help="also time the sibling dense fp16 GEMM (reported with the details)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -379,6 +385,8 @@ def main():
     if args.facts:
         hardware_facts(torch, marlin)
         return
+    if args.kernel:
+        marlin.force_kernel(args.kernel)
 
     if args.shape == "headline":
         main_name, others = "decode", ["prefill", "batch16", "mlp_up", "mlp_down", "large_g128",

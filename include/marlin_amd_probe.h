@@ -16,10 +16,12 @@ extern "C" {
 #endif
 
 /*
- * A probe launch on `stream` of device `dev`.  Kinds 0 and 1 use the grid
- * marlin_gemm uses for one row of this shape: kind 0 = an empty kernel (what a
+ * A probe launch on `stream` of device `dev`.  Kinds 0 and 1 use the grid and
+ * the workgroup size marlin_gemm uses for prob_m rows of this shape (where
+ * that is the prefill kernel's, for 16 rows): kind 0 = an empty kernel (what a
  * launch costs), kind 1 = a kernel that reads the packed weights B
- * ((prob_k/16, 2*prob_n) int32) with the streaming kernel's work split and
+ * ((prob_k/16, 2*prob_n) int32) with the work split of the kernel planned for
+ * the shape -- the streaming kernel's or the column-strip kernel's -- and
  * 128-bit loads and does nothing with them (what the weight stream alone
  * costs).  Kind 2 = a loop of nothing but v_mfma_f32_16x16x32_f16 on
  * pseudo-random operands, one workgroup of 8 waves per compute unit and
@@ -29,7 +31,8 @@ extern "C" {
  * MARLIN_OK, the marlin_gemm error code of the shape, or MARLIN_ERR_RUNTIME
  * (text in marlin_amd_probe_last_error).
  */
-int marlin_amd_probe(int kind, const void *B, int prob_n, int prob_k, int dev, void *stream);
+int marlin_amd_probe(int kind, const void *B, int prob_m, int prob_n, int prob_k, int dev,
+                     void *stream);
 
 /*
  * What a lone wave per SIMD can issue beside its MFMAs (synchronous, on the

@@ -518,7 +518,7 @@ int main(void) {
   if (marlin_official(0, 0, 0, 0, 16, 256, 0, 0, -1, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 6;
   if (marlin_gemm_static(0, 0, 0, 0, 0, 256, 512, 0, 128, 0, 0, -1, -1, -1, 16) != MARLIN_OK) return 7;
   /* the probe library beside it: an unknown kind is refused before any GPU call */
-  if (marlin_amd_probe(7, 0, 256, 512, 0, 0) != MARLIN_ERR_PROB_SHAPE) return 8;
+  if (marlin_amd_probe(7, 0, 1, 256, 512, 0, 0) != MARLIN_ERR_PROB_SHAPE) return 8;
   if (marlin_amd_probe_last_error()[0] != 0) return 9;
   printf("%s\n", marlin_amd_version());
   return 0;

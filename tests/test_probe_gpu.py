@@ -28,8 +28,17 @@ def test_launch_probes_run_and_refuse_bad_arguments(env):
     torch, marlin = env
     n, k = 1024, 1024
     B = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device="cuda")
+    assert marlin.plan(1, n, k, 128)[1]["kernel"] == 3 and marlin.plan(64, n, k, 128)[1]["kernel"] == 1
     for kind in (0, 1, 2):
-        marlin.probe(kind, B, n, k)
+        marlin.probe(kind, B, n, k)         # the column-strip kernel's split
+        marlin.probe(kind, B, n, k, m=64)   # the streaming kernel's
+        marlin.probe(kind, B, n, k, m=2048)  # prefill rows: the split of 16 rows
+    for strips in (2, 4):
+        marlin.force_strips(strips)
+        try:
+            marlin.probe(1, B, n, k)
+        finally:
+            marlin.force_strips(0)
     torch.cuda.synchronize()
     with pytest.raises(RuntimeError):
         marlin.probe(3, B, n, k)        # no such kind
