@@ -369,20 +369,24 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
 }
 
 // Fitted time (us) of the column-strip kernel with `cs` strips per workgroup,
-// at most 16 rows.  A launch costs 2.7 us; a workgroup takes in its 8 cs k
-// bytes of weights and its m rows of activations (from the L2, counted at a
-// quarter) at about 19 GB/s, what its eight waves unpack and multiply;
-// workgroups beyond one per compute unit queue up behind each other, 0.3 us
-// each; all together they draw 4.3 TB/s from memory at most.  Measured
-// (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.4, N = 11008, K = 4096
-// 8.5, N = 1024, K = 8192 6.3, 8192 x 8192 11.3 (two strips 10.8); M = 16:
-// 4096 x 4096 6.3, N = 11008, K = 4096 with four strips 10.9.
+// at most 16 rows.  A launch costs 2.7 us.  A workgroup takes in its 8 cs k
+// bytes of weights at about 23 GB/s, what its eight waves unpack and multiply,
+// and workgroups beyond one per compute unit queue up behind each other, 0.3 us
+// each; all together they draw 4.8 TB/s from memory at most.  Every workgroup
+// also reads all m rows of activations, which come from the L2s at 22 TB/s
+// together.  Measured (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.3,
+// N = 11008, K = 4096 7.8, N = 1024, K = 8192 5.5, N = 4096, K = 11008 7.5,
+// 8192 x 8192 10.4 (two strips 9.1), N = 13824, K = 5120 11.4 (four strips
+// 10.0); M = 16: 4096 x 4096 5.8, N = 11008, K = 4096 15.0 (four strips 9.4),
+// N = 4096, K = 11008 11.8.
 double strip_cost(int m, int n, int k, int cs, int cus) {
-  const int per_cu = ceil_div(n / (16 * cs), cus);
-  const double wg_bytes = 8.0 * cs * k + 0.25 * 2.0 * m * k;
-  const double by_cu = per_cu * wg_bytes / 19e3 + 0.3 * (per_cu - 1);
-  const double by_memory = 0.5 * k * n / 4.3e6;
-  return 2.7 + (by_cu > by_memory ? by_cu : by_memory);
+  const int wgs = n / (16 * cs);
+  const int per_cu = ceil_div(wgs, cus);
+  const double by_cu = per_cu * 8.0 * cs * k / 23e3;
+  const double by_memory = 0.5 * k * n / 4.8e6;
+  const double rows = wgs * 2.0 * m * k / 22e6;
+  // (a little of by_cu always: it decides between widths that memory bounds alike)
+  return 2.7 + (by_cu > by_memory ? by_cu : by_memory) + rows + 0.3 * (per_cu - 1) + 0.02 * by_cu;
 }
 
 // 16-column strips per workgroup of the column-strip kernel: the cheapest of
@@ -408,9 +412,11 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
 // share a column tile's k range, so every compute unit has work whatever n
 // is), the strips pay nothing for the exchange between workgroups -- 2 us of a
 // launch that takes 6.  The strips win while the weights are a few MiB per
-// launch (M = 1: 4096 x 4096 4.4 against 6.3 us, N = 11008, K = 4096 8.5
-// against 9.7, 8192 x 8192 10.8 against 10.4 -- there no more) and the rows
-// few (M = 16: 4096 x 4096 6.3 against 6.6, N = 11008 10.9 against 9.9).
+// launch (M = 1: 4096 x 4096 4.3 against 6.3 us, N = 11008, K = 4096 8.5
+// against 9.7, N = 4096, K = 11008 7.5 against 9.1, 8192 x 8192 9.1 against
+// 10.4, N = 28672, K = 8192 27.6 against 23.9 -- there no more) and the rows
+// few (M = 16: 4096 x 4096 5.8 against 6.6, N = 11008, K = 4096 9.4 against
+// 9.9, N = 4096, K = 11008 11.8 against 9.6).
 bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
   const int cs = strips_per_workgroup(m, n, k, cx);
   return strip_cost(m, n, k, cs, cx.cus) < stream_cost(m, n, k, cx.cus);

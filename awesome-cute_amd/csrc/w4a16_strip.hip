@@ -20,7 +20,7 @@
 // 1.4 us into the kernel instead of 0.9.
 //
 // The eight waves of a workgroup split the k range into contiguous runs of
-// chunks (256/CS k-values); each keeps two chunks in flight in registers,
+// chunks (256/CS k-values); each keeps one or two chunks in flight in registers,
 // stages the activations of a chunk through LDS into operand order by itself
 // (no barrier in the loop), and the eight partial strips are summed through
 // LDS once, at the end.  Every workgroup reads all activation rows it
@@ -279,9 +279,9 @@ template <int CS, int MR, bool GROUP>
 static int configure_strip_variant() {
   constexpr int lds = StripShape<CS, MR>::kBytes;
   if (lds <= 65536) return 0;
-  if (hipFuncSetAttribute((const void*)strip_kernel<CS, MR, GROUP, 2>,
+  if (hipFuncSetAttribute((const void*)strip_kernel<CS, MR, GROUP, 1>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess ||
-      hipFuncSetAttribute((const void*)strip_kernel<CS, MR, GROUP, 4>,
+      hipFuncSetAttribute((const void*)strip_kernel<CS, MR, GROUP, 2>,
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
     return 3;
   return 0;
@@ -305,12 +305,17 @@ static int launch_strip_variant(const GemmArgs& a, hipStream_t stream) {
   const dim3 grid(a.N / (16 * CS)), block(64 * kStripWaves);
   GemmArgs b = a;
   b.gpb = (int)grid.x;
-  // chunks in flight per wave: all of them where a wave has at most two
+  // Chunks in flight per wave: one where a wave has two at most, else two.
+  // The fewer requests the compute units have outstanding, the sooner each
+  // comes back: with everything requested at once M = 1, N = K = 4096 (two
+  // chunks per wave) took 4.36 us against 4.28, 16 rows 6.33 against 5.80;
+  // N = 4096, K = 11008 (five to six chunks per wave) 8.6 us with one chunk
+  // in flight, 7.8 with two, 8.5 with three, 9.2 with four, 9.6 with six.
   const int per_wave = ceil_div(ceil_div(a.K, StripShape<CS, MR>::kChunkK), kStripWaves);
   if (per_wave <= 2)
-    hipLaunchKernelGGL((strip_kernel<CS, MR, GROUP, 2>), grid, block, lds, stream, b);
+    hipLaunchKernelGGL((strip_kernel<CS, MR, GROUP, 1>), grid, block, lds, stream, b);
   else
-    hipLaunchKernelGGL((strip_kernel<CS, MR, GROUP, 4>), grid, block, lds, stream, b);
+    hipLaunchKernelGGL((strip_kernel<CS, MR, GROUP, 2>), grid, block, lds, stream, b);
   return launch_status();
 }
 template <int CS, bool GROUP>

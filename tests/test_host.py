@@ -219,7 +219,7 @@ def test_kernel_choice_by_cost(marlin):
     rows over small weights stream in one launch with the rows cut into parts of
     32.  The knobs override the choice."""
     for m, n, k, kernel, slices, rows in [
-            (1, 4096, 4096, 3, 1, 0), (16, 11008, 4096, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
+            (1, 4096, 4096, 3, 1, 0), (16, 4096, 11008, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
             (1, 11008, 4096, 3, 1, 0), (1, 28672, 8192, 1, 1, 0), (17, 4096, 4096, 1, 1, 0),
             (8, 2048, 2048, 3, 1, 0), (16, 8192, 8192, 1, 1, 0),
             (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 1, 1, 0),
