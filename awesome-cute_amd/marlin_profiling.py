@@ -102,7 +102,7 @@ def run_profiling(m, n, k, group_size=-1, iters=1000, model='', check=True, dev=
         'resident_us': f"{resident:.3f}",
         'hbm_us': f"{hbm:.3f}",
         'hbm_weight_GBps': f"{weight_bytes / hbm / 1e3:.0f}",
-        'kernel': 'stream' if plan['kernel'] == 1 else 'prefill',
+        'kernel': {1: 'stream', 2: 'prefill', 3: 'strips'}[plan['kernel']],
         'workgroups': plan['grid'],
         'max_rel_err': '' if err is None else f"{err:.2e}",
     }
