@@ -162,7 +162,7 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
       aq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rA, off | inv, 2 * k0, 0);
     }
     if constexpr (GROUP) {
-      int vs = (s_lane + (k0 >> 7) * p.N * 2) | inv;
+      int vs = s_lane + (valid ? (k0 >> 7) * p.N * 2 : kStripOob);
 #pragma unroll
       for (int g = 0; g < NSC; g++) {
 #pragma unroll
@@ -172,10 +172,10 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
       }
     }
     // the weights last: what comes back first is small and near
+    const int b_chunk = valid ? c * (KC * 2) * b_row : kStripOob;
 #pragma unroll
     for (int i = 0; i < 2; i++)
-      bq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
-          rB, (b_lane[i] + c * (KC * 2) * b_row) | inv, 0, 2);
+      bq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rB, b_lane[i] + b_chunk, 0, 2);
     __builtin_amdgcn_sched_barrier(0);
   };
 
