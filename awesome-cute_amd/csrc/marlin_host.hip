@@ -348,9 +348,9 @@ double stream_parts_cost(int m, int n, int k, const PlanCtx& cx, int* parts, int
   return 0.65 * (11.3 + 0.28 * *gpb) - (w == 1 ? 2.0 : 0.0);
 }
 
-bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
-  // no measurement favours 64-row prefill tiles below four row blocks
-  if (m <= 48) return false;
+// The streaming kernel's cost as make_plan would launch it: with the rows cut
+// in two or into parts of 32 where that is cheaper.
+double stream_cost_as_planned(int m, int n, int k, const PlanCtx& cx) {
   double stream = stream_cost(m, n, k, cx.cus);
   if (m <= kStreamMaxRows && cx.force.row_halves != 1 && cx.counters >= 2) {
     // what the launch gains where make_plan cuts its rows in two
@@ -365,26 +365,38 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   int parts, wpt, gpb;
   const double cut = stream_parts_cost(m, n, k, cx, &parts, &wpt, &gpb);
   if (cut > 0.0 && cut < stream) stream = cut;
-  return prefill_cost(m, n, k, cx) <= stream;
+  return stream;
+}
+
+bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
+  // no measurement favours 64-row prefill tiles below four row blocks
+  if (m <= 48) return false;
+  return prefill_cost(m, n, k, cx) <= stream_cost_as_planned(m, n, k, cx);
 }
 
 // Fitted time (us) of the column-strip kernel with `cs` strips per workgroup,
-// at most 16 rows.  A launch costs 2.7 us.  A workgroup takes in its 8 cs k
-// bytes of weights at about 23 GB/s, what its eight waves unpack and multiply,
-// and workgroups beyond one per compute unit queue up behind each other, 0.3 us
-// each; all together they draw 4.8 TB/s from memory at most.  Every workgroup
-// also reads all m rows of activations, which come from the L2s at 22 TB/s
-// together.  Measured (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.3,
+// at most 64 rows.  A launch costs 2.7 us.  A workgroup takes in its 8 cs k
+// bytes of weights at about 23 GB/s, what its eight waves unpack and multiply
+// (half as much again per row block beyond the first: more MFMAs and operand
+// reads per unpacked word), and workgroups beyond one per compute unit queue
+// up behind each other, 0.3 us each; all together they draw 4.8 TB/s from
+// memory at most.  Every workgroup also reads all rows of activations (whole
+// row blocks beyond 16 rows), which a compute unit takes from the L2s at about
+// 87 GB/s.  Measured (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.3,
 // N = 11008, K = 4096 7.8, N = 1024, K = 8192 5.5, N = 4096, K = 11008 7.5,
 // 8192 x 8192 10.4 (two strips 9.1), N = 13824, K = 5120 11.4 (four strips
 // 10.0); M = 16: 4096 x 4096 5.8, N = 11008, K = 4096 15.0 (four strips 9.4),
-// N = 4096, K = 11008 11.8.
+// N = 4096, K = 11008 11.8; M = 32: N = K = 1024 3.9, 2048 x 2048 5.2, N = 512,
+// K = 4096 7.8, 4096 x 4096 8.2; M = 64: N = 512, K = 1024 5.4, K = 4096 12.6.
 double strip_cost(int m, int n, int k, int cs, int cus) {
   const int wgs = n / (16 * cs);
   const int per_cu = ceil_div(wgs, cus);
-  const double by_cu = per_cu * 8.0 * cs * k / 23e3;
+  const int mb = ceil_div(m, 16);
+  const double by_cu = per_cu * 8.0 * cs * k / 23e3 * (1.0 + 0.5 * (mb - 1));
   const double by_memory = 0.5 * k * n / 4.8e6;
-  const double rows = wgs * 2.0 * m * k / 22e6;
+  // (with 172 of 256 compute units reading 16 rows the rows came in a third
+  // sooner than this: N = 11008, K = 4096 with four strips)
+  const double rows = per_cu * 2.0 * (mb > 1 ? 16 * mb : m) * k / 87e3 * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
   // (a little of by_cu always: it decides between widths that memory bounds alike)
   return 2.7 + (by_cu > by_memory ? by_cu : by_memory) + rows + 0.3 * (per_cu - 1) + 0.02 * by_cu;
 }
@@ -407,7 +419,7 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
   return best;
 }
 
-// The column-strip kernel against the streaming kernel for at most 16 rows:
+// The column-strip kernel against the streaming kernel for at most 64 rows:
 // the streaming kernel reaches more of the memory's bandwidth (its workgroups
 // share a column tile's k range, so every compute unit has work whatever n
 // is), the strips pay nothing for the exchange between workgroups -- 2 us of a
@@ -416,17 +428,22 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
 // against 9.7, N = 4096, K = 11008 7.5 against 9.1, 8192 x 8192 9.1 against
 // 10.4, N = 28672, K = 8192 27.6 against 23.9 -- there no more) and the rows
 // few (M = 16: 4096 x 4096 5.8 against 6.6, N = 11008, K = 4096 9.4 against
-// 9.9, N = 4096, K = 11008 11.8 against 9.6).
+// 9.9, N = 4096, K = 11008 11.8 against 9.6) or short (M = 32: N = K = 1024
+// 3.9 against 5.3, 2048 x 2048 5.2 against 5.7, N = 2048, K = 4096 8.0 against
+// 6.3; M = 64: N = 512, K = 1024 5.4 against 6.8, K = 4096 12.6 against 9.2).
 bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
   const int cs = strips_per_workgroup(m, n, k, cx);
-  return strip_cost(m, n, k, cs, cx.cus) < stream_cost(m, n, k, cx.cus);
+  // (beyond one row block the fit is looser: the strips have to win by a margin)
+  const double strips = strip_cost(m, n, k, cs, cx.cus) * (m > 16 ? 1.05 : 1.0);
+  if (strips >= stream_cost_as_planned(m, n, k, cx)) return false;
+  return !(n % 256 == 0 && m > 48 && prefill_cost(m, n, k, cx) <= strips);
 }
 
 Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   Plan pl;
-  // (the column-strip kernel does at most 16 rows and takes no hint: forced
+  // (the column-strip kernel does at most 64 rows and takes no hint: forced
   // onto anything else it leaves the choice to the costs)
-  const int force = cx.force.kernel == 3 && (m > 16 || sms > 0) ? 0 : cx.force.kernel;
+  const int force = cx.force.kernel == 3 && (m > kStripMaxRows || sms > 0) ? 0 : cx.force.kernel;
   // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
   // whenever m > 16, by the shape contract)
   const bool by_cost = force == 0 || force == 4;
@@ -437,7 +454,8 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   pl.row_parts = 1;
   pl.part_rows = 0;
   pl.strips = 0;
-  if (m <= 16 && sms <= 0 && (force == 3 || (force == 0 && prefer_strips(m, n, k, cx)))) {
+  if (m <= kStripMaxRows && sms <= 0 &&
+      (force == 3 || (force == 0 && prefer_strips(m, n, k, cx)))) {
     pl.kernel = 3;
     pl.strips = strips_per_workgroup(m, n, k, cx);
     pl.grid = n / (16 * pl.strips);

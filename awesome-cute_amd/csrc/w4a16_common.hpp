@@ -196,8 +196,10 @@ int configure_stream_kernels();
 int configure_prefill_kernels();
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
-// at most 16 rows; a workgroup per `strips` (1, 2 or 4) 16-column strips over
-// the whole k range, nothing exchanged between workgroups (w4a16_strip.hip)
+// at most kStripMaxRows rows; a workgroup per `strips` (1, 2 or 4) 16-column
+// strips over the whole k range, nothing exchanged between workgroups
+// (w4a16_strip.hip)
+constexpr int kStripMaxRows = 64;
 int configure_strip_kernels();
 int launch_strip(const GemmArgs& a, bool group, int strips, hipStream_t stream);
 // ksplit >= 1 slices of the k range per tile; above 1 the launch needs

@@ -53,7 +53,7 @@ void marlin_amd_work_order(int grid, int *out);
  * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
  * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
  * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is
- * used), 3 = the column-strip kernel (at most 16 rows and no `sms` hint, else
+ * used), 3 = the column-strip kernel (at most 64 rows and no `sms` hint, else
  * as with 0), 4 = by cost between the streaming and the prefill kernel only
  * (few rows then always meet the exchange between workgroups).  Like the overrides below it is kept per host thread, so it never
  * changes what other threads' calls do.  No reference counterpart; for tests

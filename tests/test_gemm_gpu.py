@@ -514,13 +514,17 @@ STRIP_SHAPES = [
     (5, 768, 512, 128), (8, 640, 13824, 128), (9, 1280, 1152, 128), (13, 896, 384, -1),
     (16, 256, 4096, 128), (16, 128, 128, -1), (7, 384, 640, -1), (16, 2048, 128 * 37, 128),
     (11, 1152, 64 * 2 * 51, -1), (1, 1024, 8192, -1), (16, 4096, 4096, -1), (1, 11008, 4096, 128),
+    # two to four row blocks (one weight load per chunk, the sums in the staging memory)
+    (17, 256, 256, 128), (32, 1024, 1024, 128), (33, 512, 2304, -1), (48, 768, 512, 128),
+    (64, 1024, 4096, 128), (40, 1280, 1152, 128), (64, 256, 128, -1), (50, 512, 640, -1),
+    (64, 2048, 128 * 37, 128), (31, 1280, 64 * 2 * 51, -1),
 ]
 
 
 @pytest.mark.parametrize("strips", [1, 2, 4])
 @pytest.mark.parametrize("m,n,k,g", STRIP_SHAPES)
 def test_column_strip_kernel(env, strips, m, n, k, g):
-    """The kernel for at most 16 rows whose workgroups own 16, 32 or 64 columns
+    """The kernel for at most 64 rows whose workgroups own 16, 32 or 64 columns
     over the whole k range and exchange nothing: every strip width on every
     shape, C overwritten everywhere (it starts at 9)."""
     torch, marlin = env
@@ -560,7 +564,8 @@ def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsiz
             A[np.arange(16), base + np.arange(16)] = 1.0
             C = gpu_gemm(env, A, B, sp, N)
             assert np.array_equal(C.view(np.uint16), W[base:base + 16].view(np.uint16)), base
-        for rows in ([0], [1023], [5, 700], [17, 130, 511], [3, 64, 65, 1000], list(range(2, 1024, 171))[:6]):
+        for rows in ([0], [1023], [5, 700], [17, 130, 511], [3, 64, 65, 1000], list(range(2, 1024, 171))[:6],
+                     list(range(1, 1024, 41))[:24], list(range(3, 1024, 19))[:45], list(range(0, 1024, 16))):
             A = np.zeros((len(rows), K), np.float16)
             for i, r in enumerate(rows):
                 A[i, r] = 1.0
@@ -571,13 +576,14 @@ def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsiz
         marlin.force_strips(0)
 
 
+@pytest.mark.parametrize("M", [16, 64])
 @pytest.mark.parametrize("strips", [1, 2, 4])
-def test_column_strip_kernel_closed_forms(env, strips):
+def test_column_strip_kernel_closed_forms(env, strips, M):
     """Zero point everywhere gives exact zeros; small integers times unit scales
     give exact integers (every product and every partial sum is exact in fp32)."""
     torch, marlin = env
-    M, N, K = 16, 256, 768
-    rng = np.random.default_rng(50 + strips)
+    N, K = 256, 768
+    rng = np.random.default_rng(50 + strips + M)
     marlin.force_kernel(3)
     marlin.force_strips(strips)
     try:

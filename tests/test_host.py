@@ -211,8 +211,8 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
 
 
 def test_kernel_choice_by_cost(marlin):
-    """Up to 16 rows over a few MiB of weights go through the column-strip
-    kernel, few rows otherwise through the streaming kernel, many through the prefill
+    """Up to 16 rows over a few MiB of weights, and up to 64 over a short k
+    range, go through the column-strip kernel, few rows otherwise through the streaming kernel, many through the prefill
     kernel, whose k range is cut into slices (the cheapest count, at most eight)
     while tiles alone would leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
     so do more rows while twice as many tiles save k slices; up to a few hundred
@@ -221,7 +221,8 @@ def test_kernel_choice_by_cost(marlin):
     for m, n, k, kernel, slices, rows in [
             (1, 4096, 4096, 3, 1, 0), (16, 4096, 11008, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
             (1, 11008, 4096, 3, 1, 0), (1, 28672, 8192, 1, 1, 0), (17, 4096, 4096, 1, 1, 0),
-            (8, 2048, 2048, 3, 1, 0), (16, 8192, 8192, 1, 1, 0),
+            (8, 2048, 2048, 3, 1, 0), (16, 8192, 8192, 1, 1, 0), (32, 1024, 1024, 3, 1, 0),
+            (64, 512, 1024, 3, 1, 0), (32, 2048, 4096, 1, 1, 0), (64, 512, 4096, 1, 1, 0),
             (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 1, 1, 0),
             (128, 4096, 4096, 1, 1, 0), (512, 4096, 4096, 2, 2, 64),
             (128, 8192, 8192, 2, 4, 64), (640, 4096, 11008, 2, 3, 128),
@@ -256,7 +257,8 @@ def test_kernel_choice_by_cost(marlin):
         rc, p = marlin.plan(16, 128 * 3, 512, 128, 128, 128)  # 24 strips
         assert (p["kernel"], p["strips"]) == (3, 4) and p["grid"] == 6
         marlin.force_strips(0)
-        assert marlin.plan(17, 4096, 4096, 128)[1]["kernel"] == 1  # more than 16 rows: as by cost
+        assert marlin.plan(64, 4096, 4096, 128)[1]["kernel"] == 3  # up to 64 rows
+        assert marlin.plan(65, 4096, 4096, 128)[1]["kernel"] == 1  # more: as by cost
         assert marlin.plan(2048, 4096, 4096, 128)[1]["kernel"] == 2
     finally:
         marlin.force_kernel(0)

@@ -28,11 +28,16 @@ def test_launch_probes_run_and_refuse_bad_arguments(env):
     torch, marlin = env
     n, k = 1024, 1024
     B = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device="cuda")
-    assert marlin.plan(1, n, k, 128)[1]["kernel"] == 3 and marlin.plan(64, n, k, 128)[1]["kernel"] == 1
+    assert marlin.plan(1, n, k, 128)[1]["kernel"] == 3
     for kind in (0, 1, 2):
         marlin.probe(kind, B, n, k)         # the column-strip kernel's split
-        marlin.probe(kind, B, n, k, m=64)   # the streaming kernel's
         marlin.probe(kind, B, n, k, m=2048)  # prefill rows: the split of 16 rows
+        marlin.force_kernel(4)              # (the probe library asks with the thread's overrides)
+        try:
+            assert marlin.plan(64, n, k, 128)[1]["kernel"] == 1
+            marlin.probe(kind, B, n, k, m=64)   # the streaming kernel's split
+        finally:
+            marlin.force_kernel(0)
     for strips in (2, 4):
         marlin.force_strips(strips)
         try:
