@@ -1,5 +1,5 @@
-// Column-strip W4A16 kernel for at most 16 activation rows (decode and small
-// batch): a workgroup owns 16*CS columns over the whole k range, so no two
+// Column-strip W4A16 kernel for at most 64 activation rows (decode and small
+// batch over small weights): a workgroup owns 16*CS columns over the whole k range, so no two
 // workgroups ever meet -- no partial sums in global memory, no counters, no
 // last arrival.  What that exchange costs a launch of a few microseconds
 // (store, acknowledge, ticket, read back: four trips to memory one after the
@@ -25,7 +25,7 @@
 // (no barrier in the loop), and the eight partial strips are summed through
 // LDS once, at the end.  Every workgroup reads all activation rows it
 // computes, M*K*2 bytes against 8*CS*K bytes of weights, so narrow strips pay
-// off for few rows.
+// off for few rows, and more than 16 rows only over a short k range.
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
