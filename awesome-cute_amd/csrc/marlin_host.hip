@@ -219,7 +219,9 @@ int prefill_tile_rows(int m, int n, int k, const PlanCtx& cx) {
 }
 
 double prefill_cost(int m, int n, int k, const PlanCtx& cx) {
-  return prefill_cost_rows(m, n, k, cx, prefill_tile_rows(m, n, k, cx));
+  // (the tile fits were made at K >= 4096: at K <= 1024 the prefill kernels
+  // measure a third more, 56 and 64 rows at every N from 256 to 11008)
+  return prefill_cost_rows(m, n, k, cx, prefill_tile_rows(m, n, k, cx)) * (k < 2048 ? 1.33 : 1.0);
 }
 
 // The streaming kernel's split of the granule sequence over the compute units
@@ -371,6 +373,12 @@ double stream_cost_as_planned(int m, int n, int k, const PlanCtx& cx) {
 bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   // no measurement favours 64-row prefill tiles below four row blocks
   if (m <= 48) return false;
+  // ... nor, up to 64 rows, over weights that are neither wide nor deep: 56 and
+  // 64 rows at N = 256...11008 with K = 512...4096 stream in 0.6 to 0.95 of
+  // the prefill kernel's time (N = 28672: 1.07 to 1.1 at every K; N = 11008:
+  // 1.1 at K = 8192, 1.5 at 11008), which the two fits, 15 % apart there in
+  // opposite directions, do not resolve
+  if (m <= kStreamMaxRows && n < 16384 && k < 8192) return false;
   return prefill_cost(m, n, k, cx) <= stream_cost_as_planned(m, n, k, cx);
 }
 
@@ -403,11 +411,19 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
 
 // 16-column strips per workgroup of the column-strip kernel: the cheapest of
 // 1, 2 and 4 that divide n's strips
+// (0 where the planner's own rules leave none; a forced launch takes any)
 int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
+  const bool forced = cx.force.kernel == 3 || cx.force.strips != 0;
   int best = 0;
   double best_cost = 0.0;
   for (int cs = 1; cs <= 4; cs *= 2) {
     if (n % (16 * cs) != 0) break;
+    // Several row blocks: only with a compute unit per workgroup (queued
+    // workgroups were up to 1.7 times slower than the fit: 48 rows, N = 28672)
+    // and at most two strips (with four a chunk is a single k step: N = 11008,
+    // 64 rows, K = 512...2048 1.2 to 1.3 times the streaming kernel's time
+    // where the fit promised 0.9)
+    if (m > 16 && !forced && (n / (16 * cs) > cx.cus || cs == 4)) continue;
     if (cx.force.strips != 0 && cx.force.strips != cs && best != 0) continue;
     const double c = strip_cost(m, n, k, cs, cx.cus);
     if (best == 0 || cx.force.strips == cs || c < best_cost) {
@@ -433,7 +449,10 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
 // 6.3; M = 64: N = 512, K = 1024 5.4 against 6.8, K = 4096 12.6 against 9.2).
 bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
   const int cs = strips_per_workgroup(m, n, k, cx);
-  // (beyond one row block the fit is looser: the strips have to win by a margin)
+  // (beyond one row block the fits are looser, the streaming kernel's above all
+  // over short k ranges: the strips have to win by a margin, and need a
+  // compute unit per workgroup)
+  if (cs == 0) return false;
   const double strips = strip_cost(m, n, k, cs, cx.cus) * (m > 16 ? 1.05 : 1.0);
   if (strips >= stream_cost_as_planned(m, n, k, cx)) return false;
   return !(n % 256 == 0 && m > 48 && prefill_cost(m, n, k, cx) <= strips);
@@ -791,6 +810,22 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[10] = pl.kernel == 1 ? pl.row_parts : 1;
   out[11] = pl.kernel == 1 ? pl.part_rows : 0;
   out[12] = pl.strips;
+  return rc;
+}
+
+int marlin_amd_plan_costs(int prob_m, int prob_n, int prob_k, int groupsize, int cus, double* out) {
+  for (int i = 0; i < 4; i++) out[i] = -1.0;
+  int thread_k = -1, thread_n = -1;
+  int rc = check_shape(prob_m, prob_n, prob_k, groupsize, thread_k, thread_n);
+  if (rc != MARLIN_OK || prob_m == 0 || prob_n == 0 || prob_k == 0) return rc;
+  const PlanCtx cx = {cus, kPoolPartialLimit, t_force};
+  out[0] = stream_cost_as_planned(prob_m, prob_n, prob_k, cx);
+  if (prob_n % 256 == 0) out[1] = prefill_cost(prob_m, prob_n, prob_k, cx);
+  if (prob_m <= kStripMaxRows) {
+    const int cs = strips_per_workgroup(prob_m, prob_n, prob_k, cx);
+    if (cs > 0) out[2] = strip_cost(prob_m, prob_n, prob_k, cs, cx.cus);
+    out[3] = cs;
+  }
   return rc;
 }
 

@@ -47,6 +47,8 @@ _lib.marlin_amd_force_row_halves.restype = None
 _lib.marlin_amd_force_row_halves.argtypes = [_I]
 _lib.marlin_amd_force_kernel.restype = None
 _lib.marlin_amd_force_kernel.argtypes = [_I]
+_lib.marlin_amd_plan_costs.restype = _I
+_lib.marlin_amd_plan_costs.argtypes = [_I, _I, _I, _I, _I, _P]
 _lib.marlin_amd_force_strips.restype = None
 _lib.marlin_amd_force_strips.argtypes = [_I]
 _lib.marlin_amd_work_order.restype = None
@@ -313,6 +315,14 @@ def plan(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1, sms=-1, cus=256):
     keys = ("kernel", "grid", "granules_per_wg", "col_tiles", "granules_per_tile", "launches",
             "k_slices", "tile_rows", "wgs_per_tile", "partial_kib", "row_parts", "part_rows", "strips")
     return rc, dict(zip(keys, out))
+
+
+def plan_costs(m, n, k, groupsize=-1, cus=256):
+    """The fitted costs (us) the planner compares: streaming kernel as planned, prefill kernel,
+    column strips and their width (-1 where a kernel cannot run the shape)."""
+    out = (ctypes.c_double * 4)()
+    rc = _lib.marlin_amd_plan_costs(m, n, k, groupsize, cus, out)
+    return rc, dict(zip(("stream", "prefill", "strips", "strips_per_wg"), out))
 
 
 def scratch_bytes(dev=-1):

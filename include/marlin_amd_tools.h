@@ -50,6 +50,20 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
 void marlin_amd_work_order(int grid, int *out);
 
 /*
+ * The fitted costs (microseconds on an MI355X) that the choice of kernel
+ * compares, for a device with `cus` compute units: out[0] = the streaming
+ * kernel as it would be launched (rows cut where that is cheaper), out[1] =
+ * the prefill kernel with its cheapest tile height and slice count (-1 where
+ * prob_n is no multiple of 256), out[2] = the column strips with their
+ * cheapest width and out[3] that width (-1 beyond 64 rows; cost -1 and width 0
+ * where the planner's rules allow no width).  `out` holds 4
+ * doubles.  Returns the marlin_gemm error code for the shape.  No reference
+ * counterpart; for tests and tools that check the fit against measurements.
+ */
+int marlin_amd_plan_costs(int prob_m, int prob_n, int prob_k, int groupsize, int cus,
+                          double *out);
+
+/*
  * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
  * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
  * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is

@@ -288,6 +288,30 @@ def test_kernel_choice_by_cost(marlin):
         marlin.force_tile_rows(0)
 
 
+def test_plan_costs_are_what_the_choice_compares(marlin):
+    """marlin_amd_plan_costs: the fitted costs behind the choice of kernel --
+    positive microseconds, -1 where a kernel cannot run the shape, and the plan
+    is the cheapest of them where no rule of the planner says otherwise."""
+    rc, c = marlin.plan_costs(1, 4096, 4096, 128)
+    assert rc == 0 and 3.0 < c["strips"] < c["stream"] < 8.0 and c["strips_per_wg"] == 1
+    assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 3
+    rc, c = marlin.plan_costs(2048, 4096, 4096, 128)
+    assert rc == 0 and c["strips"] == -1 and 40.0 < c["prefill"] < c["stream"]
+    rc, c = marlin.plan_costs(16, 128 * 5, 1024, 128)
+    assert rc == 0 and c["prefill"] == -1 and c["strips"] > 0      # n no multiple of 256
+    rc, c = marlin.plan_costs(32, 28672, 512, 128)
+    assert rc == 0 and c["strips"] == -1 and c["strips_per_wg"] == 0  # no width the rules allow
+    assert marlin.plan(32, 28672, 512, 128)[1]["kernel"] == 1
+    assert marlin.plan_costs(16, 100, 512, 128)[0] == 1 and marlin.plan_costs(0, 256, 512, 128)[0] == 0
+    # a short k range never takes the prefill kernel up to 64 rows, whatever the fits say
+    assert marlin.plan(64, 11008, 2048, 128)[1]["kernel"] == 1
+    for m, n, k in [(1, 11008, 4096), (16, 4096, 11008), (32, 1024, 1024), (48, 4096, 4096)]:
+        rc, c = marlin.plan_costs(m, n, k, 128)
+        margin = 1.05 if m > 16 else 1.0
+        want = 3 if c["strips"] > 0 and c["strips"] * margin < c["stream"] else 1
+        assert marlin.plan(m, n, k, 128)[1]["kernel"] == want, (m, n, k, c)
+
+
 def test_plan_picks_kernels(marlin):
     assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 3
     assert marlin.plan(32, 28672, 8192, 128)[1]["kernel"] == 1
