@@ -362,7 +362,19 @@ double stream_cost_as_planned(int m, int n, int k, const PlanCtx& cx) {
     const double gain = split.wpt >= 2 && hs.wpt >= 1 && half < m
                             ? halves_gain(m, 2 * hs.wpt, ceil_div(k / kGranuleK, 2 * hs.wpt))
                             : 0.0;
-    if (gain > 0.25) stream -= gain;
+    if (gain > 0.25) {
+      // (the halves take no less than a launch of half the rows over twice the
+      // tiles: the gain was fitted where the uncut launch fetches its sharers
+      // in rounds, which the fit of the uncut launch does not hold -- M = 64,
+      // N = 2048, K = 4096: 12.1 - 6.3 by the fits, 8.7 us measured, 8.1 by this)
+      const double alone = stream_cost(half, 2 * n, k, cx.cus);
+      stream = stream - gain > alone ? stream - gain : alone;
+    }
+    // 17 to 64 rows over short, wide weights: tiles of at most 16 granules that
+    // two to four workgroups share finish in three quarters of the fit's time
+    // (K = 512 and 1024 at N = 4096...28672: 0.6 to 0.9 of it; N <= 2048, more
+    // sharers per tile: 1.05 to 1.4)
+    if (m > 16 && k < 2048 && n >= 4096) stream *= 0.75;
   }
   int parts, wpt, gpb;
   const double cut = stream_parts_cost(m, n, k, cx, &parts, &wpt, &gpb);
@@ -382,29 +394,43 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
   return prefill_cost(m, n, k, cx) <= stream_cost_as_planned(m, n, k, cx);
 }
 
-// Fitted time (us) of the column-strip kernel with `cs` strips per workgroup,
-// at most 64 rows.  A launch costs 2.7 us.  A workgroup takes in its 8 cs k
-// bytes of weights at about 23 GB/s, what its eight waves unpack and multiply
-// (half as much again per row block beyond the first: more MFMAs and operand
-// reads per unpacked word), and workgroups beyond one per compute unit queue
-// up behind each other, 0.3 us each; all together they draw 4.8 TB/s from
-// memory at most.  Every workgroup also reads all rows of activations (whole
-// row blocks beyond 16 rows), which a compute unit takes from the L2s at about
-// 87 GB/s.  Measured (M = 1, one strip): N = K = 2048 3.2 us, 4096 x 4096 4.3,
-// N = 11008, K = 4096 7.8, N = 1024, K = 8192 5.5, N = 4096, K = 11008 7.5,
-// 8192 x 8192 10.4 (two strips 9.1), N = 13824, K = 5120 11.4 (four strips
-// 10.0); M = 16: 4096 x 4096 5.8, N = 11008, K = 4096 15.0 (four strips 9.4),
-// N = 4096, K = 11008 11.8; M = 32: N = K = 1024 3.9, 2048 x 2048 5.2, N = 512,
-// K = 4096 7.8, 4096 x 4096 8.2; M = 64: N = 512, K = 1024 5.4, K = 4096 12.6.
+// Fitted time (us) of the column-strip kernel with `cs` strips per workgroup.
+// Up to 16 rows a launch costs 2.7 us.  A workgroup takes in its 8 cs k bytes
+// of weights at about 23 GB/s, what its eight waves unpack and multiply, and
+// workgroups beyond one per compute unit queue up behind each other, 0.3 us
+// each; all together they draw 4.8 TB/s from memory at most.  Every workgroup
+// also reads all rows of activations, which a compute unit takes from the L2s
+// at about 87 GB/s.  Measured (M = 1, one strip): N = K = 2048 3.2 us, 4096 x
+// 4096 4.3, N = 11008, K = 4096 7.8, N = 1024, K = 8192 5.5, N = 4096, K =
+// 11008 7.5, 8192 x 8192 10.4 (two strips 9.1), N = 13824, K = 5120 11.4 (four
+// strips 10.0); M = 16: 4096 x 4096 5.8, N = 11008, K = 4096 15.0 (four strips
+// 9.4), N = 4096, K = 11008 11.8.
+// More rows are cut into parts of 16, a workgroup per strip set and part, and
+// fitted on their own: 1.8 us, and per round of workgroups over the compute
+// units 1.27 us, the weights at 32.7 GB/s and the part's 16 rows at 67.8 GB/s,
+// a quarter of which later rounds hide behind the one before.  Measured: M =
+// 32, N = K = 1024 3.9 us, 2048 x 2048 4.6, 4096 x 4096 7.6; M = 64: N = 512,
+// K = 1024 3.6, N = 2048, K = 4096 7.7, 4096 x 4096 9.7; M = 128: N = 256, K =
+// 512 3.4, 2048 x 2048 6.8; M = 512: N = 256, K = 1024 3.7; M = 1024: N =
+// 256, K = 512 3.8.
 double strip_cost(int m, int n, int k, int cs, int cus) {
+  const double by_memory = 0.5 * k * n / 4.8e6;
+  if (m > 16) {
+    // rows in parts of 16, a workgroup each: fitted to 17...128 rows over N =
+    // 256...28672, K = 512...11008 (8 % rms where the strips are within 1.6
+    // times the other kernels' time)
+    const int wgs = n / (16 * cs) * ceil_div(m, 16);
+    const int rounds = ceil_div(wgs, cus);
+    const double per_wg = 1.27 + 8.0 * cs * k / 32.7e3 + 32.0 * k / 67.8e3;
+    const double by_cu = rounds * per_wg * (1.0 - 0.24 * (1.0 - 1.0 / rounds));
+    return 1.8 + (by_cu > by_memory ? by_cu : by_memory);
+  }
   const int wgs = n / (16 * cs);
   const int per_cu = ceil_div(wgs, cus);
-  const int mb = ceil_div(m, 16);
-  const double by_cu = per_cu * 8.0 * cs * k / 23e3 * (1.0 + 0.5 * (mb - 1));
-  const double by_memory = 0.5 * k * n / 4.8e6;
+  const double by_cu = per_cu * 8.0 * cs * k / 23e3;
   // (with 172 of 256 compute units reading 16 rows the rows came in a third
   // sooner than this: N = 11008, K = 4096 with four strips)
-  const double rows = per_cu * 2.0 * (mb > 1 ? 16 * mb : m) * k / 87e3 * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
+  const double rows = per_cu * 2.0 * m * k / 87e3 * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
   // (a little of by_cu always: it decides between widths that memory bounds alike)
   return 2.7 + (by_cu > by_memory ? by_cu : by_memory) + rows + 0.3 * (per_cu - 1) + 0.02 * by_cu;
 }
@@ -423,7 +449,12 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
     // and at most two strips (with four a chunk is a single k step: N = 11008,
     // 64 rows, K = 512...2048 1.2 to 1.3 times the streaming kernel's time
     // where the fit promised 0.9)
-    if (m > 16 && !forced && (n / (16 * cs) > cx.cus || cs == 4)) continue;
+    // Rows in parts: at most two workgroups per compute unit (with three and
+    // more the streaming kernel was 1.1 to 1.6 times faster wherever the fits,
+    // its own 20 to 40 % high over short k ranges, promised otherwise: 48 rows
+    // at N = 28672, K = 512 11.8 against 7.3 us, 64 rows at N = 11008, K = 2048
+    // 13.5 against 11.2)
+    if (m > 16 && !forced && n / (16 * cs) * ceil_div(m, 16) > 2 * cx.cus) continue;
     if (cx.force.strips != 0 && cx.force.strips != cs && best != 0) continue;
     const double c = strip_cost(m, n, k, cs, cx.cus);
     if (best == 0 || cx.force.strips == cs || c < best_cost) {
@@ -435,23 +466,27 @@ int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
   return best;
 }
 
-// The column-strip kernel against the streaming kernel for at most 64 rows:
-// the streaming kernel reaches more of the memory's bandwidth (its workgroups
-// share a column tile's k range, so every compute unit has work whatever n
-// is), the strips pay nothing for the exchange between workgroups -- 2 us of a
-// launch that takes 6.  The strips win while the weights are a few MiB per
-// launch (M = 1: 4096 x 4096 4.3 against 6.3 us, N = 11008, K = 4096 8.5
-// against 9.7, N = 4096, K = 11008 7.5 against 9.1, 8192 x 8192 9.1 against
-// 10.4, N = 28672, K = 8192 27.6 against 23.9 -- there no more) and the rows
-// few (M = 16: 4096 x 4096 5.8 against 6.6, N = 11008, K = 4096 9.4 against
-// 9.9, N = 4096, K = 11008 11.8 against 9.6) or short (M = 32: N = K = 1024
-// 3.9 against 5.3, 2048 x 2048 5.2 against 5.7, N = 2048, K = 4096 8.0 against
-// 6.3; M = 64: N = 512, K = 1024 5.4 against 6.8, K = 4096 12.6 against 9.2).
+// The column-strip kernel against the other two: the streaming kernel reaches
+// more of the memory's bandwidth (its workgroups share a column tile's k
+// range, so every compute unit has work whatever n is), the strips pay nothing
+// for the exchange between workgroups -- 2 us of a launch that takes 6.  The
+// strips win while the weights are a few MiB per launch (M = 1: 4096 x 4096
+// 4.3 against 6.3 us, N = 11008, K = 4096 8.5 against 9.7, N = 4096, K = 11008
+// 7.5 against 9.1, 8192 x 8192 9.1 against 10.4, N = 28672, K = 8192 27.6
+// against 23.9 -- there no more; M = 16: 4096 x 4096 5.8 against 6.6, N =
+// 11008, K = 4096 9.4 against 9.9, N = 4096, K = 11008 11.8 against 9.6), and
+// with more rows, in parts, while the parts fill the compute units at most
+// twice (M = 32: N = K = 1024 3.9 against 5.6, 4096 x 4096 7.6 against 8.5, N =
+// 8192, K = 4096 9.5 against 10.3, N = 4096, K = 8192 11.0 against 10.7; M =
+// 64: N = 512, K = 1024 3.6 against 6.9, N = 2048, K = 4096 7.7 against 8.7,
+// 4096 x 4096 9.7 against 10.5, N = 8192, K = 4096 15.0 against 13.3; M =
+// 128: N = 256, K = 512 3.4 against 7.0, 2048 x 2048 6.8 against 8.1, 4096 x
+// 4096 14.6 against 12.9; M = 1024: N = 256, K = 512 3.8 against 7.7, N = 512,
+// K = 1024 6.6 against 11.4).
 bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
   const int cs = strips_per_workgroup(m, n, k, cx);
   // (beyond one row block the fits are looser, the streaming kernel's above all
-  // over short k ranges: the strips have to win by a margin, and need a
-  // compute unit per workgroup)
+  // over short k ranges: the strips have to win by a margin)
   if (cs == 0) return false;
   const double strips = strip_cost(m, n, k, cs, cx.cus) * (m > 16 ? 1.05 : 1.0);
   if (strips >= stream_cost_as_planned(m, n, k, cx)) return false;
@@ -460,8 +495,8 @@ bool prefer_strips(int m, int n, int k, const PlanCtx& cx) {
 
 Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
   Plan pl;
-  // (the column-strip kernel does at most 64 rows and takes no hint: forced
-  // onto anything else it leaves the choice to the costs)
+  // (the column-strip kernel does at most kStripMaxRows rows and takes no
+  // hint: forced onto anything else it leaves the choice to the costs)
   const int force = cx.force.kernel == 3 && (m > kStripMaxRows || sms > 0) ? 0 : cx.force.kernel;
   // the prefill kernel's tiles are 256 columns wide (n is a multiple of 256
   // whenever m > 16, by the shape contract)
@@ -477,7 +512,11 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
       (force == 3 || (force == 0 && prefer_strips(m, n, k, cx)))) {
     pl.kernel = 3;
     pl.strips = strips_per_workgroup(m, n, k, cx);
-    pl.grid = n / (16 * pl.strips);
+    if (m > 16) {
+      pl.row_parts = ceil_div(m, 16);
+      pl.part_rows = 16;
+    }
+    pl.grid = n / (16 * pl.strips) * pl.row_parts;
     pl.sp = make_stream_plan(n, k, 1);
     pl.launches = 1;
     return pl;
@@ -572,6 +611,7 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
   int rc = MARLIN_OK;
   if (pl.kernel == 3) {
     GemmArgs a;
+    const int strip_parts = pl.row_parts;
     a.A = A;
     a.B = B;
     a.C = C;
@@ -584,8 +624,8 @@ int enqueue(const Plan& pl, const ScratchView& view, const void* A, const void* 
     a.scratch = nullptr;
     a.gpb = 0;
     a.wpt = 0;
-    a.row_parts = 1;
-    a.part_rows = 0;
+    a.row_parts = strip_parts;
+    a.part_rows = strip_parts > 1 ? 16 : 0;
     rc = launch_strip(a, groupsize != -1, pl.strips, stream);
   } else if (pl.kernel == 2) {
     GemmArgs a;
@@ -807,8 +847,8 @@ int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int threa
   out[7] = pl.tile_rows;
   out[8] = pl.kernel == 1 ? pl.sp.wpt : 0;
   out[9] = (int)(pl.partial_bytes >> 10);
-  out[10] = pl.kernel == 1 ? pl.row_parts : 1;
-  out[11] = pl.kernel == 1 ? pl.part_rows : 0;
+  out[10] = pl.kernel == 1 || pl.kernel == 3 ? pl.row_parts : 1;
+  out[11] = pl.kernel == 1 || pl.kernel == 3 ? pl.part_rows : 0;
   out[12] = pl.strips;
   return rc;
 }

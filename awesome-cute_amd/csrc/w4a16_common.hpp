@@ -173,7 +173,8 @@ struct GemmArgs {
   int row_parts;    // streaming kernel, wpt > 0: 1, or the number of parts the rows are cut
                     // into, `part_rows` each (the last one the rest), that separate
                     // workgroups compute: wpt workgroups per column tile and part; needs
-                    // lock_stride >= row_parts
+                    // lock_stride >= row_parts.  Column-strip kernel: 1, or the number
+                    // of 16-row parts, a workgroup per strip set and part
   int part_rows;    // rows of a part: 16 or 32
 };
 
@@ -196,10 +197,10 @@ int configure_stream_kernels();
 int configure_prefill_kernels();
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
-// at most kStripMaxRows rows; a workgroup per `strips` (1, 2 or 4) 16-column
-// strips over the whole k range, nothing exchanged between workgroups
-// (w4a16_strip.hip)
-constexpr int kStripMaxRows = 64;
+// at most kStripMaxRows rows, 16 x a.row_parts at most; a workgroup per
+// `strips` (1, 2 or 4) 16-column strips and 16-row part over the whole k range,
+// nothing exchanged between workgroups (w4a16_strip.hip)
+constexpr int kStripMaxRows = 1024;
 int configure_strip_kernels();
 int launch_strip(const GemmArgs& a, bool group, int strips, hipStream_t stream);
 // ksplit >= 1 slices of the k range per tile; above 1 the launch needs

@@ -86,7 +86,8 @@ __global__ __launch_bounds__(512) void probe_read_strips_kernel(GemmArgs p, int*
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int wid = xcd_work_index((int)blockIdx.x, (int)gridDim.x);
-  const int strip0 = wid * CS;
+  // (rows in parts: every part of a strip set reads the set's weights)
+  const int strip0 = (p.row_parts > 1 ? wid / p.row_parts : wid) * CS;
   const int n_chunks = ceil_div(p.K, 16 * kRows);
   const int c0 = (wave * n_chunks) / 8, c1 = ((wave + 1) * n_chunks) / 8;
   const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
@@ -328,6 +329,7 @@ int marlin_amd_probe(int kind, const void* B, int prob_m, int prob_n, int prob_k
     a.M = 1;
     a.N = prob_n;
     a.K = prob_k;
+    a.row_parts = plan[10];
     if (strips == 1)
       hipLaunchKernelGGL(probe_read_strips_kernel<1>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
     else if (strips == 2)

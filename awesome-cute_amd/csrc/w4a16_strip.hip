@@ -1,7 +1,7 @@
-// Column-strip W4A16 kernel for at most 64 activation rows (decode and small
-// batch over small weights): a workgroup owns 16*CS columns over the whole k range, so no two
-// workgroups ever meet -- no partial sums in global memory, no counters, no
-// last arrival.  What that exchange costs a launch of a few microseconds
+// Column-strip W4A16 kernel, 16 activation rows per workgroup (decode, small
+// batches, and more rows over small weights): a workgroup owns 16*CS columns
+// over the whole k range, so no two workgroups ever meet -- no partial sums in
+// global memory, no counters, no last arrival.  What that exchange costs a launch of a few microseconds
 // (store, acknowledge, ticket, read back: four trips to memory one after the
 // other) is more than what narrow strips cost the weight stream.
 //
@@ -25,7 +25,18 @@
 // (no barrier in the loop), and the eight partial strips are summed through
 // LDS once, at the end.  Every workgroup reads all activation rows it
 // computes, M*K*2 bytes against 8*CS*K bytes of weights, so narrow strips pay
-// off for few rows, and more than 16 rows only over a short k range.
+// off for few rows.
+//
+// More than 16 rows are cut into parts of 16, each a workgroup of its own over
+// the same strips: grid = strip sets x parts.  The parts of a strip set have
+// neighbouring work indices (one L2), so the weights come from memory once and
+// from the L2 for the other parts; every part unpacks them again, which a
+// launch of a few microseconds over small weights can afford.  (Several row
+// blocks inside one workgroup, sharing every unpacked weight, were slower
+// wherever they were tried: a workgroup then reads 16 x row blocks rows of
+// activations, and eight waves' rows of a chunk fill LDS.  M = 64: N = 2048,
+// K = 4096 12.9 us with four row blocks per workgroup, 7.0 in parts; N = 512,
+// K = 1024 5.4 / 3.6; N = K = 4096 13.1 / 9.5.)
 #include "w4a16_common.hpp"
 
 namespace w4a16 {
@@ -42,57 +53,38 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t strip_rsrc(const void* p, unsi
 }  // namespace
 
 // CS: 16-column strips per workgroup (1, 2 or 4: a 64-column block at most).
-// MR: activation rows staged (2, 4, 8, 16, 32, 48 or 64; rows past M are read
-// as zeros): MB = ceil(MR / 16) row blocks share every unpacked weight.
-// A chunk is what one wave requests at a time: two weight loads (eight rows of
-// a strip each, 256/CS k-values together) with one row block, one weight load
-// with more -- the activations of a chunk pass through LDS, and 64 rows of 256
-// k-values for each of eight waves would not fit.
+// MR: activation rows staged (2, 4, 8 or 16; rows past M are read as zeros).
 template <int CS, int MR>
 struct StripShape {
-  static constexpr int kRowBlocks = (MR + 15) / 16;
-  static constexpr int kWeightLoads = MR <= 16 ? 2 : 1;  // per chunk
-  static constexpr int kStepsPerLoad = 4 / CS;           // 32-deep k steps in a weight load
-  static constexpr int kSteps = kWeightLoads * kStepsPerLoad;
-  static constexpr int kChunkK = 32 * kSteps;            // k-values per chunk
-  static constexpr int kRowBytes = 2 * kChunkK;          // of one activation row per chunk
+  static constexpr int kSteps = 8 / CS;               // 32-deep k steps per chunk
+  static constexpr int kChunkK = 32 * kSteps;         // k-values per chunk
+  static constexpr int kRowBytes = 2 * kChunkK;       // of one activation row per chunk
   static constexpr int kLanesPerRow = kRowBytes / 16;
   static constexpr int kRowsPerLoad = 64 / kLanesPerRow;
   static constexpr int kALoads = (MR + kRowsPerLoad - 1) / kRowsPerLoad;
   static constexpr int kRowsStaged = kALoads * kRowsPerLoad;
   // 16 bytes of padding per row: MFMA lanes (kg, row) then read 64 distinct banks
   static constexpr int kStride = kRowBytes + 16;
-  // per wave: the activation rows of a chunk, then its 1 or 2 KiB of weights
+  // per wave: the activation rows of a chunk, then its 2 KiB of weights
   static constexpr int kWeightBase = kRowsStaged * kStride;
-  static constexpr int kStagePerWave = kWeightBase + 1024 * kWeightLoads;
-  static constexpr int kStageBytes = kStripWaves * kStagePerWave;
-  static constexpr int kReduceBytes = kStripWaves * CS * kRowBlocks * 1024;
-  // With one row block the cross-wave sums have LDS of their own; with more
-  // they reuse the staging memory, behind a barrier.
-  static constexpr bool kReduceInStage = kRowBlocks > 1;
-  static constexpr int kReduceBase = kReduceInStage ? 0 : kStageBytes;
-  static constexpr int kBytes = kReduceInStage
-                                    ? (kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes)
-                                    : kStageBytes + kReduceBytes;
-  static_assert(kBytes <= 160 * 1024, "LDS of a compute unit");
-  static_assert(kRowsStaged >= 16 * kRowBlocks || kRowBlocks == 1, "whole row blocks are staged");
+  static constexpr int kStagePerWave = kWeightBase + 2048;
+  static constexpr int kReduceBase = kStripWaves * kStagePerWave;
+  static constexpr int kBytes = kReduceBase + kStripWaves * CS * 1024;
 };
 
 template <int CS, int MR, bool GROUP, int DEPTH>
 __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   using Sh = StripShape<CS, MR>;
   constexpr int KC = Sh::kSteps;
-  constexpr int KH = Sh::kStepsPerLoad;
-  constexpr int NB = Sh::kWeightLoads;
-  constexpr int MB = Sh::kRowBlocks;
-  constexpr int NSC = GROUP ? (Sh::kChunkK > 128 ? 2 : 1) : 0;  // scale rows a chunk touches
+  constexpr int NSC = GROUP ? (CS == 1 ? 2 : 1) : 0;  // scale rows a chunk touches
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   {
     // all kernel arguments in one trip to memory, ahead of the first load
     const void *a_ = p.A, *b_ = p.B, *s_ = p.S;
     void* c_ = p.C;
-    asm volatile("" ::"s"(a_), "s"(b_), "s"(s_), "s"(c_), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.gpb));
+    asm volatile("" ::"s"(a_), "s"(b_), "s"(s_), "s"(c_), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.gpb),
+                 "s"(p.row_parts));
   }
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -101,7 +93,11 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   const int nu = lane & 15;
   // (p.gpb carries the grid: the launch's own record of it is a second trip to memory)
   const int wid = xcd_work_index((int)blockIdx.x, p.gpb);
-  const int strip0 = wid * CS;  // my first strip; strip S holds bytes [128 S, 128 S + 128) of a row of B
+  // rows in parts (p.row_parts > 1): work index w computes rows [16 part, 16
+  // part + 16) of strip set w / row_parts, part = w % row_parts
+  const int set = p.row_parts > 1 ? wid / p.row_parts : wid;
+  const int row0 = p.row_parts > 1 ? 16 * (wid - set * p.row_parts) : 0;
+  const int strip0 = set * CS;  // my first strip; strip S holds bytes [128 S, 128 S + 128) of a row of B
 
   // my chunks [c0, c1) of the k range
   const int n_chunks = ceil_div(p.K, Sh::kChunkK);
@@ -114,12 +110,12 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
       strip_rsrc(p.S, (unsigned)(GROUP ? p.K / 128 : 1) * (unsigned)p.N * 2u);
   const int b_row = p.N * 8;  // bytes per row of B
 
-  // weights, fetched: the 64 lanes of a weight load take 16 bytes each in the
-  // order [row][strip][Marlin lane] (8/CS rows; a chunk's second load the next
-  // 8/CS); used: word j = (nu/2)%4 of Marlin lane (t = kg, c = 2s + e), e = nu/8
-  int b_lane[NB];
+  // weights, fetched: the 128 lanes of a chunk's two loads take 16 bytes each
+  // in the order [row][strip][Marlin lane]; used: word j = (nu/2)%4 of Marlin
+  // lane (t = kg, c = 2s + e), e = nu/8
+  int b_lane[2];
 #pragma unroll
-  for (int i = 0; i < NB; i++) {
+  for (int i = 0; i < 2; i++) {
     const int idx = 64 * i + lane;
     b_lane[i] = (idx / (8 * CS)) * b_row + 128 * (strip0 + (idx / 8) % CS) + 16 * (idx % 8);
   }
@@ -136,40 +132,33 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
 #pragma unroll
   for (int i = 0; i < Sh::kALoads; i++) {
     const int r = i * Sh::kRowsPerLoad + a_row;
-    a_lane[i] = r < p.M ? r * p.K * 2 + 16 * a_piece : kStripOob;
+    a_lane[i] = row0 + r < p.M ? (row0 + r) * p.K * 2 + 16 * a_piece : kStripOob;
   }
   char* stage = smem + wave * Sh::kStagePerWave;
   const int a_wr = a_row * Sh::kStride + 16 * a_piece;
-  // MFMA lane (kg, row nu) of row block i reads dwords kg, kg+4, kg+8, kg+12 of
-  // the 64 bytes of row 16i + nu and its k step; rows that are not staged read
-  // row 0 (never stored)
+  // MFMA lane (kg, row nu) reads dwords kg, kg+4, kg+8, kg+12 of the 64 bytes
+  // of its row and k step; rows that are not staged read row 0 (never stored)
   const int a_rd = (nu < Sh::kRowsStaged ? nu : 0) * Sh::kStride + 4 * kg;
 
-  // The cross-wave sums have CS * MB items (strip s, row block i), number
-  // s * MB + i; wave w writes items w and w + 8.  Result lane (row m = lane%16,
-  // q = lane/16) holds in register r the column slot nu = 4q + r, i.e. e = q/2,
-  // j = 2(q%2) + r/2, h = r%2: column 16j + 8h + 2s' + e of the block, s' the
-  // strip's place in the block.  The per-channel scales of those columns are
-  // fetched now.
-  constexpr int kItems = CS * MB;
-  constexpr int kItemsPerWave = (kItems + kStripWaves - 1) / kStripWaves;
-  const int res_col = 64 * (strip0 >> 2) + 2 * (strip0 & 3) + 32 * (kg & 1) + (kg >> 1);
-  unsigned short chan[kItemsPerWave][4];
+  // Result lane (row m = lane%16, q = lane/16) holds in register r the column
+  // slot nu = 4q + r, i.e. e = q/2, j = 2(q%2) + r/2, h = r%2: column
+  // 16j + 8h + 2s' + e of the block, s' the strip's place in the block.  The
+  // per-channel scales of those columns are fetched now (wave s < CS writes
+  // strip s in the end).
+  const int res_col = 64 * (strip0 >> 2) + 2 * (strip0 & 3) + 32 * (kg & 1) + (kg >> 1) + 2 * wave;
+  unsigned short chan[4] = {0, 0, 0, 0};
   if constexpr (!GROUP) {
-#pragma unroll
-    for (int t = 0; t < kItemsPerWave; t++) {
-      const int item = wave + kStripWaves * t;
-      const int s = item < kItems ? item / MB : 0;
+    if (wave < CS) {
 #pragma unroll
       for (int r = 0; r < 4; r++)
-        chan[t][r] = __builtin_amdgcn_raw_buffer_load_b16(
-            rS, 2 * scale_index_single(res_col + 2 * s + 16 * (r >> 1) + 8 * (r & 1)), 0, 0);
+        chan[r] = __builtin_amdgcn_raw_buffer_load_b16(
+            rS, 2 * scale_index_single(res_col + 16 * (r >> 1) + 8 * (r & 1)), 0, 0);
     }
   }
 
   const DequantConsts dc;
 
-  i4 bq[DEPTH][NB];
+  i4 bq[DEPTH][2];
   unsigned short sq[DEPTH][NSC > 0 ? NSC * CS : 1];
   i4 aq[DEPTH][Sh::kALoads];
 
@@ -201,104 +190,69 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
     // the weights last: what comes back first is small and near
     const int b_chunk = valid ? c * (KC * 2) * b_row : kStripOob;
 #pragma unroll
-    for (int i = 0; i < NB; i++)
+    for (int i = 0; i < 2; i++)
       bq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rB, b_lane[i] + b_chunk, 0, 2);
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  f4 acc[CS][MB][2];
+  f4 acc[CS][2];
 #pragma unroll
-  for (int s = 0; s < CS; s++)
-#pragma unroll
-    for (int i = 0; i < MB; i++) acc[s][i][0] = acc[s][i][1] = (f4){0.f, 0.f, 0.f, 0.f};
-
-  const h2 sub = {(half_t)1032.f, (half_t)1032.f};
-  const h2 mul = {(half_t)0.0625f, (half_t)0.0625f};
-  const h2 add = {(half_t)-72.f, (half_t)-72.f};
-  // k step q of the chunk in LDS: the operand of row block i, the two packed
-  // words (rows 2q and 2q+1) of strip s, and the MFMAs of the step
-  auto read_a = [&](int q, int i) {
-    const int* ap = (const int*)(stage + a_rd + i * 16 * Sh::kStride + 64 * q);
-    return (i4){ap[0], ap[4], ap[8], ap[12]};
-  };
-  auto read_w = [&](int q, int s, int x) {
-    const int* wp = (const int*)(stage + Sh::kWeightBase + (2 * q * CS + s) * 128 + b_rd);
-    return wp[32 * CS * x];
-  };
-  auto step = [&](int slot, int q, const i4 (&av)[MB], const int (&wv)[CS][2]) {
-#pragma unroll
-    for (int s = 0; s < CS; s++) {
-      const int wa = (int)((unsigned)wv[s][0] >> shift);
-      const int wb = (int)((unsigned)wv[s][1] >> shift);
-      h2 la = as_h2((wa & dc.lo_mask) | dc.ex) - sub;
-      h2 ha = __builtin_elementwise_fma(as_h2((wa & dc.hi_mask) | dc.ex), mul, add);
-      h2 lb = as_h2((wb & dc.lo_mask) | dc.ex) - sub;
-      h2 hb = __builtin_elementwise_fma(as_h2((wb & dc.hi_mask) | dc.ex), mul, add);
-      if constexpr (GROUP) {
-        const int g = NSC == 2 ? q / 4 : 0;
-        const half_t sc = __builtin_bit_cast(half_t, sq[slot][g * CS + s]);
-        const h2 s2 = {sc, sc};
-        la *= s2;
-        ha *= s2;
-        lb *= s2;
-        hb *= s2;
-      }
-      const h8 w = make_h8(la, ha, lb, hb);
-#pragma unroll
-      for (int i = 0; i < MB; i++)
-        acc[s][i][q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-            w, __builtin_bit_cast(h8, av[i]), acc[s][i][q & 1], 0, 0, 0);
-    }
-  };
+  for (int s = 0; s < CS; s++) acc[s][0] = acc[s][1] = (f4){0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](int slot) {
     // activations of the chunk: registers -> LDS, rows as they are
 #pragma unroll
     for (int i = 0; i < Sh::kALoads; i++)
       *(i4*)(stage + i * Sh::kRowsPerLoad * Sh::kStride + a_wr) = aq[slot][i];
-    // Each weight load of the chunk is used as it lands: registers -> LDS as
-    // fetched ([row][strip][Marlin lane]), then its k steps.  With one row
-    // block all operands of the load come back from LDS before the first is
-    // used (read one k step at a time, every step would wait out a trip to
-    // LDS); with more, a step's operands are read while the step before it
-    // multiplies.
+    const h2 sub = {(half_t)1032.f, (half_t)1032.f};
+    const h2 mul = {(half_t)0.0625f, (half_t)0.0625f};
+    const h2 add = {(half_t)-72.f, (half_t)-72.f};
+    // Each of the chunk's two weight loads holds half its k steps and is used
+    // as it lands: registers -> LDS as fetched ([row][strip][Marlin lane]),
+    // then all operands of the half back from LDS before the first of them is
+    // used (read one k step at a time, every step would wait out a trip to LDS).
+    constexpr int KH = KC / 2;
 #pragma unroll
-    for (int half = 0; half < NB; half++) {
+    for (int half = 0; half < 2; half++) {
       *(i4*)(stage + Sh::kWeightBase + (64 * half + lane) * 16) = bq[slot][half];
-      if constexpr (MB == 1) {
-        i4 av[KH][1];
-        int wv[KH][CS][2];
+      i4 av[KH];
+      int wv[KH][CS][2];
 #pragma unroll
-        for (int u = 0; u < KH; u++) {
-          const int q = half * KH + u;
-          av[u][0] = read_a(q, 0);
+      for (int u = 0; u < KH; u++) {
+        const int q = half * KH + u;
+        const int* ap = (const int*)(stage + a_rd + 64 * q);
+        av[u] = (i4){ap[0], ap[4], ap[8], ap[12]};
 #pragma unroll
-          for (int s = 0; s < CS; s++) {
-            wv[u][s][0] = read_w(q, s, 0);
-            wv[u][s][1] = read_w(q, s, 1);
-          }
+        for (int s = 0; s < CS; s++) {
+          const int* wp = (const int*)(stage + Sh::kWeightBase + (2 * q * CS + s) * 128 + b_rd);
+          wv[u][s][0] = wp[0];
+          wv[u][s][1] = wp[32 * CS];
         }
-        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < KH; u++) step(slot, half * KH + u, av[u], wv[u]);
-      } else {
-        i4 av[2][MB];
-        int wv[2][CS][2];
-        auto fetch = [&](int u) {
-          const int q = half * KH + u;
+      for (int u = 0; u < KH; u++) {
+        const int q = half * KH + u;
+        const h8 af = __builtin_bit_cast(h8, av[u]);
 #pragma unroll
-          for (int i = 0; i < MB; i++) av[u & 1][i] = read_a(q, i);
-#pragma unroll
-          for (int s = 0; s < CS; s++) {
-            wv[u & 1][s][0] = read_w(q, s, 0);
-            wv[u & 1][s][1] = read_w(q, s, 1);
+        for (int s = 0; s < CS; s++) {
+          const int wa = (int)((unsigned)wv[u][s][0] >> shift);
+          const int wb = (int)((unsigned)wv[u][s][1] >> shift);
+          h2 la = as_h2((wa & dc.lo_mask) | dc.ex) - sub;
+          h2 ha = __builtin_elementwise_fma(as_h2((wa & dc.hi_mask) | dc.ex), mul, add);
+          h2 lb = as_h2((wb & dc.lo_mask) | dc.ex) - sub;
+          h2 hb = __builtin_elementwise_fma(as_h2((wb & dc.hi_mask) | dc.ex), mul, add);
+          if constexpr (GROUP) {
+            const int g = CS == 1 ? q / 4 : 0;
+            const half_t sc = __builtin_bit_cast(half_t, sq[slot][g * CS + s]);
+            const h2 s2 = {sc, sc};
+            la *= s2;
+            ha *= s2;
+            lb *= s2;
+            hb *= s2;
           }
-        };
-        fetch(0);
-#pragma unroll
-        for (int u = 0; u < KH; u++) {
-          if (u + 1 < KH) fetch(u + 1);
-          step(slot, half * KH + u, av[u & 1], wv[u & 1]);
+          acc[s][q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(make_h8(la, ha, lb, hb), af,
+                                                                 acc[s][q & 1], 0, 0, 0);
         }
       }
     }
@@ -314,30 +268,23 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
     }
   }
 
-  // ---- sum the eight waves
+  // ---- sum the eight waves; wave s < CS writes strip s
   f4* red = (f4*)(smem + Sh::kReduceBase);
-  if constexpr (Sh::kReduceInStage) __syncthreads();  // every wave is done with its staging
 #pragma unroll
-  for (int s = 0; s < CS; s++)
-#pragma unroll
-    for (int i = 0; i < MB; i++)
-      red[((wave * CS + s) * MB + i) * 64 + lane] = acc[s][i][0] + acc[s][i][1];
+  for (int s = 0; s < CS; s++) red[(wave * CS + s) * 64 + lane] = acc[s][0] + acc[s][1];
   __syncthreads();
+  if (wave < CS) {
+    const int s = wave;
+    f4 v = red[s * 64 + lane];
 #pragma unroll
-  for (int t = 0; t < kItemsPerWave; t++) {
-    const int item = wave + kStripWaves * t;
-    if (item >= kItems) break;
-    const int s = item / MB, i = item - s * MB;
-    f4 v = red[item * 64 + lane];
-#pragma unroll
-    for (int w = 1; w < kStripWaves; w++) v += red[(w * kItems + item) * 64 + lane];
-    const int m = 16 * i + nu;
+    for (int w = 1; w < kStripWaves; w++) v += red[(w * CS + s) * 64 + lane];
+    const int m = row0 + nu;
     if (m < p.M) {
-      half_t* crow = (half_t*)p.C + (size_t)m * p.N + res_col + 2 * s;
+      half_t* crow = (half_t*)p.C + (size_t)m * p.N + res_col;
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         half_t o = (half_t)v[r];
-        if constexpr (!GROUP) o *= __builtin_bit_cast(half_t, chan[t][r]);
+        if constexpr (!GROUP) o *= __builtin_bit_cast(half_t, chan[r]);
         crow[16 * (r >> 1) + 8 * (r & 1)] = o;
       }
     }
@@ -355,16 +302,12 @@ static int configure_strip_variant() {
     return 3;
   return 0;
 }
-template <int CS, int MR>
-static int configure_strip_rows() {
-  return configure_strip_variant<CS, MR, false>() | configure_strip_variant<CS, MR, true>();
-}
 template <int CS>
 static int configure_strip_width() {
-  return configure_strip_rows<CS, 2>() | configure_strip_rows<CS, 4>() |
-         configure_strip_rows<CS, 8>() | configure_strip_rows<CS, 16>() |
-         configure_strip_rows<CS, 32>() | configure_strip_rows<CS, 48>() |
-         configure_strip_rows<CS, 64>();
+  return configure_strip_variant<CS, 2, false>() | configure_strip_variant<CS, 2, true>() |
+         configure_strip_variant<CS, 4, false>() | configure_strip_variant<CS, 4, true>() |
+         configure_strip_variant<CS, 8, false>() | configure_strip_variant<CS, 8, true>() |
+         configure_strip_variant<CS, 16, false>() | configure_strip_variant<CS, 16, true>();
 }
 
 int configure_strip_kernels() {
@@ -375,7 +318,7 @@ int configure_strip_kernels() {
 template <int CS, int MR, bool GROUP>
 static int launch_strip_variant(const GemmArgs& a, hipStream_t stream) {
   constexpr int lds = StripShape<CS, MR>::kBytes;
-  const dim3 grid(a.N / (16 * CS)), block(64 * kStripWaves);
+  const dim3 grid(a.N / (16 * CS) * (a.row_parts > 1 ? a.row_parts : 1)), block(64 * kStripWaves);
   GemmArgs b = a;
   b.gpb = (int)grid.x;
   // Chunks in flight per wave: one where a wave has two at most, else two.
@@ -393,18 +336,17 @@ static int launch_strip_variant(const GemmArgs& a, hipStream_t stream) {
 }
 template <int CS, bool GROUP>
 static int launch_strip_rows(const GemmArgs& a, hipStream_t stream) {
+  if (a.row_parts > 1) return launch_strip_variant<CS, 16, GROUP>(a, stream);  // parts of 16 rows
   if (a.M <= 2) return launch_strip_variant<CS, 2, GROUP>(a, stream);
   if (a.M <= 4) return launch_strip_variant<CS, 4, GROUP>(a, stream);
   if (a.M <= 8) return launch_strip_variant<CS, 8, GROUP>(a, stream);
-  if (a.M <= 16) return launch_strip_variant<CS, 16, GROUP>(a, stream);
-  if (a.M <= 32) return launch_strip_variant<CS, 32, GROUP>(a, stream);
-  if (a.M <= 48) return launch_strip_variant<CS, 48, GROUP>(a, stream);
-  return launch_strip_variant<CS, 64, GROUP>(a, stream);
+  return launch_strip_variant<CS, 16, GROUP>(a, stream);
 }
 
 // strips: 16-column strips per workgroup (1, 2 or 4; N a multiple of 16*strips)
 int launch_strip(const GemmArgs& a, bool group, int strips, hipStream_t stream) {
-  if (a.M > kStripMaxRows || a.N % (16 * strips) != 0) return 2;
+  const int parts = a.row_parts > 1 ? a.row_parts : 1;
+  if (a.M > 16 * parts || a.M > kStripMaxRows || a.N % (16 * strips) != 0) return 2;
   switch (strips * 2 + (group ? 1 : 0)) {
     case 2: return launch_strip_rows<1, false>(a, stream);
     case 3: return launch_strip_rows<1, true>(a, stream);

@@ -273,7 +273,7 @@ def check(m, n, k, groupsize=-1, thread_k=-1, thread_n=-1):
 
 def force_kernel(which):
     """0 = choose by cost, 1 = streaming kernel, 2 = prefill kernel, 3 = column-strip kernel
-    (at most 64 rows; other problems are planned as with 0), 4 = by cost without the
+    (at most 1024 rows; other problems are planned as with 0), 4 = by cost without the
     column-strip kernel -- calling thread only."""
     _lib.marlin_amd_force_kernel(int(which))
 

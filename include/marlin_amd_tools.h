@@ -33,7 +33,9 @@ int marlin_amd_check(int prob_m, int prob_n, int prob_k, int groupsize, int thre
  * exchanges through the library's scratch (0 = none); out[10] = parts the
  * streaming kernel cuts the rows into (1 = uncut; every part is a problem of
  * its own for out[8] workgroups per column tile), out[11] = rows of a part;
- * out[12] = 16-column strips per workgroup of the column-strip kernel (else 0).
+ * out[12] = 16-column strips per workgroup of the column-strip kernel (else 0),
+ * which cuts more than 16 rows into out[10] parts of 16, a workgroup per strip
+ * set and part (out[1] = strip sets x parts).
  * `out` holds 13 ints.  Returns the marlin_gemm error code for the shape.
  */
 int marlin_amd_plan(int prob_m, int prob_n, int prob_k, int groupsize, int thread_k,
@@ -55,7 +57,7 @@ void marlin_amd_work_order(int grid, int *out);
  * kernel as it would be launched (rows cut where that is cheaper), out[1] =
  * the prefill kernel with its cheapest tile height and slice count (-1 where
  * prob_n is no multiple of 256), out[2] = the column strips with their
- * cheapest width and out[3] that width (-1 beyond 64 rows; cost -1 and width 0
+ * cheapest width and out[3] that width (-1 beyond 1024 rows; cost -1 and width 0
  * where the planner's rules allow no width).  `out` holds 4
  * doubles.  Returns the marlin_gemm error code for the shape.  No reference
  * counterpart; for tests and tools that check the fit against measurements.
@@ -67,10 +69,11 @@ int marlin_amd_plan_costs(int prob_m, int prob_n, int prob_k, int groupsize, int
  * Which kernel marlin_gemm uses for calls made by the calling thread: 0 =
  * choose by cost (default), 1 = the streaming kernel, 64 rows per launch, 2 =
  * the prefill kernel (needs prob_n % 256 == 0, else the streaming kernel is
- * used), 3 = the column-strip kernel (at most 64 rows and no `sms` hint, else
- * as with 0), 4 = by cost between the streaming and the prefill kernel only
- * (few rows then always meet the exchange between workgroups).  Like the overrides below it is kept per host thread, so it never
- * changes what other threads' calls do.  No reference counterpart; for tests
+ * used), 3 = the column-strip kernel (at most 1024 rows and no `sms` hint,
+ * else as with 0), 4 = by cost between the streaming and the prefill kernel
+ * only (few rows then always meet the exchange between workgroups).  Like the
+ * overrides below it is kept per host thread, so it never changes what other
+ * threads' calls do.  No reference counterpart; for tests
  * and tools.
  */
 void marlin_amd_force_kernel(int which);

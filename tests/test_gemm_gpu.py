@@ -514,25 +514,29 @@ STRIP_SHAPES = [
     (5, 768, 512, 128), (8, 640, 13824, 128), (9, 1280, 1152, 128), (13, 896, 384, -1),
     (16, 256, 4096, 128), (16, 128, 128, -1), (7, 384, 640, -1), (16, 2048, 128 * 37, 128),
     (11, 1152, 64 * 2 * 51, -1), (1, 1024, 8192, -1), (16, 4096, 4096, -1), (1, 11008, 4096, 128),
-    # two to four row blocks (one weight load per chunk, the sums in the staging memory)
+    # more rows in parts of 16, a workgroup per strip set and part: whole and ragged
+    # last parts, more workgroups than compute units, the most rows the kernel takes
     (17, 256, 256, 128), (32, 1024, 1024, 128), (33, 512, 2304, -1), (48, 768, 512, 128),
     (64, 1024, 4096, 128), (40, 1280, 1152, 128), (64, 256, 128, -1), (50, 512, 640, -1),
-    (64, 2048, 128 * 37, 128), (31, 1280, 64 * 2 * 51, -1),
+    (64, 2048, 128 * 37, 128), (31, 1280, 64 * 2 * 51, -1), (128, 512, 1024, 128),
+    (97, 768, 640, -1), (250, 2048, 512, 128), (513, 512, 640, -1), (1024, 256, 512, 128),
 ]
 
 
 @pytest.mark.parametrize("strips", [1, 2, 4])
 @pytest.mark.parametrize("m,n,k,g", STRIP_SHAPES)
 def test_column_strip_kernel(env, strips, m, n, k, g):
-    """The kernel for at most 64 rows whose workgroups own 16, 32 or 64 columns
-    over the whole k range and exchange nothing: every strip width on every
-    shape, C overwritten everywhere (it starts at 9)."""
+    """The kernel whose workgroups own 16, 32 or 64 columns (and 16 rows) over
+    the whole k range and exchange nothing: every strip width on every shape,
+    C overwritten everywhere (it starts at 9)."""
     torch, marlin = env
     marlin.force_kernel(3)
     marlin.force_strips(strips)
     try:
         rc, p = marlin.plan(m, n, k, g)
-        assert (rc, p["kernel"], p["strips"], p["grid"]) == (0, 3, strips, n // (16 * strips))
+        parts = -(-m // 16)
+        assert (rc, p["kernel"], p["strips"], p["row_parts"]) == (0, 3, strips, parts)
+        assert p["grid"] == n // (16 * strips) * parts and p["launches"] == 1 and p["partial_kib"] == 0
         A, q, s, B, sp = O.make_problem(m, n, k, g, seed=m + n + k)
         C = gpu_gemm(env, A, B, sp, n, C_fill=9.0)
     finally:
@@ -549,7 +553,8 @@ def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsiz
     """One-hot rows through the column strips return the dequantised weights bit
     for bit: every k of a 1024-deep weight (16 rows at a time: all staged-row
     counts' widest instance), then single rows and short batches (the narrower
-    instances), for every strip width and both scale modes."""
+    instances) and batches of several 16-row parts, for every strip width and
+    both scale modes."""
     torch, marlin = env
     N, K = 256, 1024
     _, q, s, B, sp = O.make_problem(1, N, K, groupsize, seed=13)
@@ -565,7 +570,8 @@ def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsiz
             C = gpu_gemm(env, A, B, sp, N)
             assert np.array_equal(C.view(np.uint16), W[base:base + 16].view(np.uint16)), base
         for rows in ([0], [1023], [5, 700], [17, 130, 511], [3, 64, 65, 1000], list(range(2, 1024, 171))[:6],
-                     list(range(1, 1024, 41))[:24], list(range(3, 1024, 19))[:45], list(range(0, 1024, 16))):
+                     list(range(1, 1024, 41))[:24], list(range(3, 1024, 19))[:45], list(range(0, 1024, 16)),
+                     list(range(1, 1024, 5))[:200]):
             A = np.zeros((len(rows), K), np.float16)
             for i, r in enumerate(rows):
                 A[i, r] = 1.0
@@ -576,7 +582,7 @@ def test_column_strip_kernel_dequantized_weights_bit_exact(env, strips, groupsiz
         marlin.force_strips(0)
 
 
-@pytest.mark.parametrize("M", [16, 64])
+@pytest.mark.parametrize("M", [16, 64, 200])
 @pytest.mark.parametrize("strips", [1, 2, 4])
 def test_column_strip_kernel_closed_forms(env, strips, M):
     """Zero point everywhere gives exact zeros; small integers times unit scales
@@ -608,7 +614,8 @@ def test_few_rows_through_either_kernel_agree_with_the_oracle(env):
     """The shapes the planner gives to the column strips, through the streaming
     kernel as well: both inside the tolerance, on the same inputs."""
     torch, marlin = env
-    for (m, n, k, g) in [(1, 4096, 4096, 128), (8, 2048, 2048, -1), (16, 1280, 1152, 128)]:
+    for (m, n, k, g) in [(1, 4096, 4096, 128), (8, 2048, 2048, -1), (16, 1280, 1152, 128),
+                         (64, 1024, 1024, 128), (200, 512, 1024, -1)]:
         assert marlin.plan(m, n, k, g)[1]["kernel"] == 3
         for which in (0, 4):
             marlin.force_kernel(which)

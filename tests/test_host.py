@@ -211,20 +211,22 @@ def test_default_stream_plans_stay_inside_tiles(marlin, m, n, k):
 
 
 def test_kernel_choice_by_cost(marlin):
-    """Up to 16 rows over a few MiB of weights, and up to 64 over a short k
-    range, go through the column-strip kernel, few rows otherwise through the streaming kernel, many through the prefill
-    kernel, whose k range is cut into slices (the cheapest count, at most eight)
+    """Up to 16 rows over a few MiB of weights, and more rows (in parts of 16,
+    a workgroup each) while the parts fill the compute units at most twice, go
+    through the column-strip kernel, few rows otherwise through the streaming
+    kernel, many through the prefill kernel, whose k range is cut into slices (the cheapest count, at most eight)
     while tiles alone would leave CUs idle; 49-64 rows over big weights take 64-row prefill tiles, and
     so do more rows while twice as many tiles save k slices; up to a few hundred
     rows over small weights stream in one launch with the rows cut into parts of
     32.  The knobs override the choice."""
     for m, n, k, kernel, slices, rows in [
             (1, 4096, 4096, 3, 1, 0), (16, 4096, 11008, 1, 1, 0), (48, 28672, 8192, 1, 1, 0),
-            (1, 11008, 4096, 3, 1, 0), (1, 28672, 8192, 1, 1, 0), (17, 4096, 4096, 1, 1, 0),
+            (1, 11008, 4096, 3, 1, 0), (1, 28672, 8192, 1, 1, 0), (17, 4096, 4096, 3, 1, 0),
             (8, 2048, 2048, 3, 1, 0), (16, 8192, 8192, 1, 1, 0), (32, 1024, 1024, 3, 1, 0),
-            (64, 512, 1024, 3, 1, 0), (32, 2048, 4096, 1, 1, 0), (64, 512, 4096, 1, 1, 0),
-            (64, 4096, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64), (96, 4096, 4096, 1, 1, 0),
-            (128, 4096, 4096, 1, 1, 0), (512, 4096, 4096, 2, 2, 64),
+            (64, 512, 1024, 3, 1, 0), (32, 2048, 4096, 3, 1, 0), (64, 512, 4096, 3, 1, 0),
+            (64, 4096, 4096, 3, 1, 0), (64, 8192, 4096, 1, 1, 0), (64, 28672, 8192, 2, 2, 64),
+            (96, 4096, 4096, 1, 1, 0), (128, 4096, 4096, 1, 1, 0), (128, 512, 1024, 3, 1, 0),
+            (1024, 256, 512, 3, 1, 0), (1040, 256, 512, 2, 1, 64), (512, 4096, 4096, 2, 2, 64),
             (128, 8192, 8192, 2, 4, 64), (640, 4096, 11008, 2, 3, 128),
             (512, 4096, 11008, 2, 4, 128), (1024, 4096, 4096, 2, 2, 128),
             (1536, 4096, 4096, 2, 1, 128), (2048, 4096, 4096, 2, 1, 128)]:
@@ -237,8 +239,8 @@ def test_kernel_choice_by_cost(marlin):
     rc, p = marlin.plan(128, 4096, 4096, 128)
     assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 4, 32, 2)
     assert p["grid"] == 32 * 4 * 2
-    rc, p = marlin.plan(64, 4096, 4096, 128)
-    assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 2, 32, 4)
+    rc, p = marlin.plan(64, 8192, 4096, 128)
+    assert (p["launches"], p["row_parts"], p["part_rows"], p["wgs_per_tile"]) == (1, 2, 32, 2)
     rc, p = marlin.plan(16, 4096, 11008, 128)
     assert (p["kernel"], p["row_parts"], p["wgs_per_tile"], p["strips"]) == (1, 1, 8, 0)
     # column strips: a workgroup per 16, 32 or 64 columns, nothing exchanged, one launch
@@ -246,6 +248,11 @@ def test_kernel_choice_by_cost(marlin):
     assert (p["kernel"], p["strips"], p["grid"], p["launches"], p["partial_kib"]) == (3, 1, 256, 1, 0)
     rc, p = marlin.plan(1, 8192, 1024, 128)
     assert (p["kernel"], p["strips"], p["grid"]) == (3, 2, 256)
+    # ... and per 16 rows: strip sets x parts
+    rc, p = marlin.plan(64, 4096, 4096, 128)
+    assert (p["kernel"], p["strips"], p["row_parts"], p["part_rows"], p["grid"]) == (3, 4, 4, 16, 256)
+    rc, p = marlin.plan(100, 512, 1024, 128)
+    assert (p["kernel"], p["strips"], p["row_parts"], p["grid"], p["launches"]) == (3, 1, 7, 32 * 7, 1)
     assert marlin.plan(1, 4096, 4096, 128, sms=64)[1]["kernel"] == 1  # a hint asks for the streaming split
     try:
         marlin.force_kernel(3)
@@ -257,8 +264,9 @@ def test_kernel_choice_by_cost(marlin):
         rc, p = marlin.plan(16, 128 * 3, 512, 128, 128, 128)  # 24 strips
         assert (p["kernel"], p["strips"]) == (3, 4) and p["grid"] == 6
         marlin.force_strips(0)
-        assert marlin.plan(64, 4096, 4096, 128)[1]["kernel"] == 3  # up to 64 rows
-        assert marlin.plan(65, 4096, 4096, 128)[1]["kernel"] == 1  # more: as by cost
+        rc, p = marlin.plan(1024, 4096, 4096, 128)  # up to 1024 rows
+        assert (p["kernel"], p["row_parts"], p["grid"]) == (3, 64, 64 * 4096 // (16 * p["strips"]))
+        assert marlin.plan(1025, 4096, 4096, 128)[1]["kernel"] == 2  # more: as by cost
         assert marlin.plan(2048, 4096, 4096, 128)[1]["kernel"] == 2
     finally:
         marlin.force_kernel(0)
@@ -269,7 +277,7 @@ def test_kernel_choice_by_cost(marlin):
         assert rc == 0 and p["kernel"] == 1 and p["launches"] == 32 and p["row_parts"] == 1
         marlin.force_kernel(2)
         rc, p = marlin.plan(100, 512, 1024, 128)
-        assert rc == 0 and p["kernel"] == 2
+        assert rc == 0 and p["kernel"] == 2 and p["row_parts"] == 1
         assert p["grid"] == -(-100 // p["tile_rows"]) * 2 * p["k_slices"]
         marlin.force_tile_rows(128)
         assert marlin.plan(100, 512, 1024, 128)[1]["tile_rows"] == 128
@@ -300,12 +308,14 @@ def test_plan_costs_are_what_the_choice_compares(marlin):
     rc, c = marlin.plan_costs(16, 128 * 5, 1024, 128)
     assert rc == 0 and c["prefill"] == -1 and c["strips"] > 0      # n no multiple of 256
     rc, c = marlin.plan_costs(32, 28672, 512, 128)
-    assert rc == 0 and c["strips"] == -1 and c["strips_per_wg"] == 0  # no width the rules allow
+    assert rc == 0 and c["strips"] == -1 and c["strips_per_wg"] == 0  # no width the rules allow:
+    # parts of 16 rows may fill the compute units twice, no more (2 x 448 workgroups with four strips)
     assert marlin.plan(32, 28672, 512, 128)[1]["kernel"] == 1
     assert marlin.plan_costs(16, 100, 512, 128)[0] == 1 and marlin.plan_costs(0, 256, 512, 128)[0] == 0
     # a short k range never takes the prefill kernel up to 64 rows, whatever the fits say
     assert marlin.plan(64, 11008, 2048, 128)[1]["kernel"] == 1
-    for m, n, k in [(1, 11008, 4096), (16, 4096, 11008), (32, 1024, 1024), (48, 4096, 4096)]:
+    for m, n, k in [(1, 11008, 4096), (16, 4096, 11008), (32, 1024, 1024), (48, 4096, 4096),
+                    (64, 8192, 4096), (32, 4096, 8192), (128, 2048, 2048), (256, 512, 4096)]:
         rc, c = marlin.plan_costs(m, n, k, 128)
         margin = 1.05 if m > 16 else 1.0
         want = 3 if c["strips"] > 0 and c["strips"] * margin < c["stream"] else 1

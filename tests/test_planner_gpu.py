@@ -2,7 +2,7 @@
 dozen shapes from the decode to the prefill regime, the planned launch must not
 be more than 10 % slower than the best of the forced alternatives -- the
 streaming kernel, the prefill kernel on 64-row tiles and on 128-row tiles, each
-with the slice count its cost model picks, and for at most 64 rows the
+with the slice count its cost model picks, and for at most 1024 rows the
 column-strip kernel with 1, 2 and 4 strips per workgroup (for at most 16 rows
 instead of the prefill kernel).  The planner is a fitted cost model;
 this test is what fails when a kernel change shifts the costs under it.  (The
@@ -23,9 +23,11 @@ SHAPES = [(m, n, k) for (n, k) in [(4096, 4096), (4096, 11008), (8192, 8192)]
 SHAPES += [(m, n, k) for (n, k) in [(4096, 4096), (11008, 4096), (4096, 11008), (2048, 2048),
                                     (8192, 8192), (1024, 8192)]
            for m in (1, 16)]
-# 17 to 64 rows over small weights: column strips where the k range is short
+# more rows over small weights: column strips, the rows in parts of 16, while the
+# parts fill the compute units at most twice
 SHAPES += [(32, 1024, 1024), (64, 512, 1024), (32, 2048, 2048), (33, 512, 2048), (32, 2048, 4096),
-           (64, 512, 4096), (48, 1024, 4096)]
+           (64, 512, 4096), (48, 1024, 4096), (64, 8192, 4096), (128, 512, 1024), (128, 2048, 2048),
+           (96, 4096, 2048), (256, 1024, 1024), (1024, 256, 512), (512, 512, 2048)]
 SLACK = 1.10
 
 
@@ -84,7 +86,7 @@ def _measure(torch, marlin, m, n, k):
         times["planned"] = _us_per_call(torch, call, 40)
         marlin.force_kernel(1)
         times["streaming"] = _us_per_call(torch, call, 40)
-        if m <= 64:
+        if m <= 1024:
             for strips in (1, 2, 4):
                 marlin.force_kernel(3)
                 marlin.force_strips(strips)

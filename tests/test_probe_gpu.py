@@ -32,6 +32,8 @@ def test_launch_probes_run_and_refuse_bad_arguments(env):
     for kind in (0, 1, 2):
         marlin.probe(kind, B, n, k)         # the column-strip kernel's split
         marlin.probe(kind, B, n, k, m=2048)  # prefill rows: the split of 16 rows
+        assert marlin.plan(64, n, k, 128)[1]["row_parts"] == 4
+        marlin.probe(kind, B, n, k, m=64)   # column strips, the rows in four parts
         marlin.force_kernel(4)              # (the probe library asks with the thread's overrides)
         try:
             assert marlin.plan(64, n, k, 128)[1]["kernel"] == 1
