@@ -139,7 +139,7 @@ constexpr int kStreamMaxRows = 64;
 struct Force {
   int kernel = 0, k_slices = 0, tile_rows = 0;
   int row_halves = 0;  // streaming kernel: 0 = by cost, 1 = never cut the rows, 2 = cut them where possible
-  int strips = 0;      // column-strip kernel: 0 = by cost, or 1, 2, 4 strips per workgroup
+  int strips = 0;      // column-strip kernel: 0 = by cost, or 1 to 4 strips per workgroup
 };
 thread_local Force t_force;
 
@@ -419,13 +419,13 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
     // rows in parts of 16, a workgroup each: fitted to 17...128 rows over N =
     // 256...28672, K = 512...11008 (8 % rms where the strips are within 1.6
     // times the other kernels' time)
-    const int wgs = n / (16 * cs) * ceil_div(m, 16);
+    const int wgs = ceil_div(n / 16, cs) * ceil_div(m, 16);
     const int rounds = ceil_div(wgs, cus);
     const double per_wg = 1.27 + 8.0 * cs * k / 32.7e3 + 32.0 * k / 67.8e3;
     const double by_cu = rounds * per_wg * (1.0 - 0.24 * (1.0 - 1.0 / rounds));
     return 1.8 + (by_cu > by_memory ? by_cu : by_memory);
   }
-  const int wgs = n / (16 * cs);
+  const int wgs = ceil_div(n / 16, cs);
   const int per_cu = ceil_div(wgs, cus);
   const double by_cu = per_cu * 8.0 * cs * k / 23e3;
   // (with 172 of 256 compute units reading 16 rows the rows came in a third
@@ -436,25 +436,24 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
 }
 
 // 16-column strips per workgroup of the column-strip kernel: the cheapest of
-// 1, 2 and 4 that divide n's strips
+// 1, 2 and 4 where they divide n's strips, and for up to 16 rows of 3, which
+// leaves the last workgroup with fewer (N = 11008, K = 4096, 230 workgroups
+// of three strips against 172 of four: M = 16 9.2 against 9.3 us, M = 8 8.2 /
+// 8.5, M = 1 7.5 / 7.7 with one strip; N = 5120, K = 5120: 10.3 against 8.4
+// with two)
 // (0 where the planner's own rules leave none; a forced launch takes any)
 int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
   const bool forced = cx.force.kernel == 3 || cx.force.strips != 0;
   int best = 0;
   double best_cost = 0.0;
-  for (int cs = 1; cs <= 4; cs *= 2) {
-    if (n % (16 * cs) != 0) break;
-    // Several row blocks: only with a compute unit per workgroup (queued
-    // workgroups were up to 1.7 times slower than the fit: 48 rows, N = 28672)
-    // and at most two strips (with four a chunk is a single k step: N = 11008,
-    // 64 rows, K = 512...2048 1.2 to 1.3 times the streaming kernel's time
-    // where the fit promised 0.9)
+  for (int cs = 1; cs <= 4; cs++) {
+    if (cs == 3 ? (m > 16 && !forced) : n % (16 * cs) != 0) continue;
     // Rows in parts: at most two workgroups per compute unit (with three and
     // more the streaming kernel was 1.1 to 1.6 times faster wherever the fits,
     // its own 20 to 40 % high over short k ranges, promised otherwise: 48 rows
     // at N = 28672, K = 512 11.8 against 7.3 us, 64 rows at N = 11008, K = 2048
     // 13.5 against 11.2)
-    if (m > 16 && !forced && n / (16 * cs) * ceil_div(m, 16) > 2 * cx.cus) continue;
+    if (m > 16 && !forced && ceil_div(n / 16, cs) * ceil_div(m, 16) > 2 * cx.cus) continue;
     if (cx.force.strips != 0 && cx.force.strips != cs && best != 0) continue;
     const double c = strip_cost(m, n, k, cs, cx.cus);
     if (best == 0 || cx.force.strips == cs || c < best_cost) {
@@ -516,7 +515,7 @@ Plan make_plan(int m, int n, int k, int sms, const PlanCtx& cx) {
       pl.row_parts = ceil_div(m, 16);
       pl.part_rows = 16;
     }
-    pl.grid = n / (16 * pl.strips) * pl.row_parts;
+    pl.grid = ceil_div(n / 16, pl.strips) * pl.row_parts;
     pl.sp = make_stream_plan(n, k, 1);
     pl.launches = 1;
     return pl;
@@ -871,7 +870,7 @@ int marlin_amd_plan_costs(int prob_m, int prob_n, int prob_k, int groupsize, int
 
 void marlin_amd_force_kernel(int which) { t_force.kernel = which >= 1 && which <= 4 ? which : 0; }
 void marlin_amd_force_strips(int strips) {
-  t_force.strips = strips == 1 || strips == 2 || strips == 4 ? strips : 0;
+  t_force.strips = strips >= 1 && strips <= 4 ? strips : 0;
 }
 
 void marlin_amd_force_k_slices(int slices) { t_force.k_slices = slices > 0 ? slices : 0; }

@@ -198,7 +198,7 @@ int configure_prefill_kernels();
 
 int launch_stream(const GemmArgs& a, bool group, int grid, hipStream_t stream);
 // at most kStripMaxRows rows, 16 x a.row_parts at most; a workgroup per
-// `strips` (1, 2 or 4) 16-column strips and 16-row part over the whole k range,
+// `strips` (1 to 4) 16-column strips and 16-row part over the whole k range,
 // nothing exchanged between workgroups (w4a16_strip.hip)
 constexpr int kStripMaxRows = 1024;
 int configure_strip_kernels();

@@ -81,7 +81,9 @@ __global__ __launch_bounds__(256) void probe_read_kernel(GemmArgs p, int* sink) 
 
 template <int CS>
 __global__ __launch_bounds__(512) void probe_read_strips_kernel(GemmArgs p, int* sink) {
-  constexpr int kRows = 16 / CS;  // rows of B per chunk: two loads of 1 KiB per wave
+  // rows of B per chunk: two loads of 1 KiB per wave (three for three strips)
+  constexpr int NL = CS == 3 ? 3 : 2;
+  constexpr int kRows = 8 * NL / CS;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
@@ -93,18 +95,22 @@ __global__ __launch_bounds__(512) void probe_read_strips_kernel(GemmArgs p, int*
   const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<void*>(p.B), 0, (int)((unsigned)p.K * (unsigned)(p.N / 2)), 0x00020000);
   const int b_row = p.N * 8;
-  int b_lane[2];
+  int b_lane[NL];
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < NL; i++) {
     const int idx = 64 * i + lane;
-    b_lane[i] = (idx / (8 * CS)) * b_row + 128 * (strip0 + (idx / 8) % CS) + 16 * (idx % 8);
+    const int strip = strip0 + (idx / 8) % CS;
+    // (a strip past the last one, of a last workgroup of three, is not read)
+    b_lane[i] = strip < (p.N >> 4)
+                    ? (idx / (8 * CS)) * b_row + 128 * strip + 16 * (idx % 8)
+                    : kProbeOob;
   }
   i4 acc = {0, 0, 0, 0};
-  i4 buf[kProbeDepth][2];
+  i4 buf[kProbeDepth][NL];
   auto issue = [&](int slot, int c) {
     const int inv = c < c1 ? 0 : kProbeOob;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NL; i++)
       buf[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
           rB, (b_lane[i] + c * kRows * b_row) | inv, 0, 2);
   };
@@ -113,7 +119,8 @@ __global__ __launch_bounds__(512) void probe_read_strips_kernel(GemmArgs p, int*
   for (int c = c0; c < c1; c += kProbeDepth) {
 #pragma unroll
     for (int d = 0; d < kProbeDepth; d++) {
-      acc |= buf[d][0] | buf[d][1];
+#pragma unroll
+      for (int i = 0; i < NL; i++) acc |= buf[d][i];
       issue(d, c + d + kProbeDepth);
     }
   }
@@ -334,6 +341,8 @@ int marlin_amd_probe(int kind, const void* B, int prob_m, int prob_n, int prob_k
       hipLaunchKernelGGL(probe_read_strips_kernel<1>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
     else if (strips == 2)
       hipLaunchKernelGGL(probe_read_strips_kernel<2>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
+    else if (strips == 3)
+      hipLaunchKernelGGL(probe_read_strips_kernel<3>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
     else
       hipLaunchKernelGGL(probe_read_strips_kernel<4>, dim3(grid), dim3(512), 0, stream, a, (int*)nullptr);
   } else if (kind == 1) {

@@ -52,11 +52,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t strip_rsrc(const void* p, unsi
 
 }  // namespace
 
-// CS: 16-column strips per workgroup (1, 2 or 4: a 64-column block at most).
+// CS: 16-column strips per workgroup (1 to 4; three where N's strips fill the
+// compute units better in threes, the last workgroup then with fewer).
 // MR: activation rows staged (2, 4, 8 or 16; rows past M are read as zeros).
 template <int CS, int MR>
 struct StripShape {
-  static constexpr int kSteps = 8 / CS;               // 32-deep k steps per chunk
+  // a chunk is two weight loads of 1 KiB per wave (three for three strips): 16
+  // (24) lines of 128 bytes, CS lines per row of B, two rows per k step
+  static constexpr int kLoads = CS == 3 ? 3 : 2;
+  static constexpr int kSteps = 4 * kLoads / CS;      // 32-deep k steps per chunk
   static constexpr int kChunkK = 32 * kSteps;         // k-values per chunk
   static constexpr int kRowBytes = 2 * kChunkK;       // of one activation row per chunk
   static constexpr int kLanesPerRow = kRowBytes / 16;
@@ -65,9 +69,9 @@ struct StripShape {
   static constexpr int kRowsStaged = kALoads * kRowsPerLoad;
   // 16 bytes of padding per row: MFMA lanes (kg, row) then read 64 distinct banks
   static constexpr int kStride = kRowBytes + 16;
-  // per wave: the activation rows of a chunk, then its 2 KiB of weights
+  // per wave: the activation rows of a chunk, then its 2 (3) KiB of weights
   static constexpr int kWeightBase = kRowsStaged * kStride;
-  static constexpr int kStagePerWave = kWeightBase + 2048;
+  static constexpr int kStagePerWave = kWeightBase + 1024 * kLoads;
   static constexpr int kReduceBase = kStripWaves * kStagePerWave;
   static constexpr int kBytes = kReduceBase + kStripWaves * CS * 1024;
 };
@@ -76,6 +80,7 @@ template <int CS, int MR, bool GROUP, int DEPTH>
 __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   using Sh = StripShape<CS, MR>;
   constexpr int KC = Sh::kSteps;
+  constexpr int NL = Sh::kLoads;
   constexpr int NSC = GROUP ? (CS == 1 ? 2 : 1) : 0;  // scale rows a chunk touches
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -98,6 +103,7 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   const int set = p.row_parts > 1 ? wid / p.row_parts : wid;
   const int row0 = p.row_parts > 1 ? 16 * (wid - set * p.row_parts) : 0;
   const int strip0 = set * CS;  // my first strip; strip S holds bytes [128 S, 128 S + 128) of a row of B
+  const int n_strips = p.N >> 4;  // (three strips per workgroup: the last one may hold fewer)
 
   // my chunks [c0, c1) of the k range
   const int n_chunks = ceil_div(p.K, Sh::kChunkK);
@@ -110,14 +116,17 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
       strip_rsrc(p.S, (unsigned)(GROUP ? p.K / 128 : 1) * (unsigned)p.N * 2u);
   const int b_row = p.N * 8;  // bytes per row of B
 
-  // weights, fetched: the 128 lanes of a chunk's two loads take 16 bytes each
+  // weights, fetched: the 128 (192) lanes of a chunk's loads take 16 bytes each
   // in the order [row][strip][Marlin lane]; used: word j = (nu/2)%4 of Marlin
   // lane (t = kg, c = 2s + e), e = nu/8
-  int b_lane[2];
+  int b_lane[NL];
+  bool b_mine[NL];  // (a strip past the last one would be the next row's first)
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < NL; i++) {
     const int idx = 64 * i + lane;
-    b_lane[i] = (idx / (8 * CS)) * b_row + 128 * (strip0 + (idx / 8) % CS) + 16 * (idx % 8);
+    const int strip = strip0 + (idx / 8) % CS;
+    b_lane[i] = (idx / (8 * CS)) * b_row + 128 * strip + 16 * (idx % 8);
+    b_mine[i] = CS != 3 || strip < n_strips;
   }
   const int b_rd = (4 * (nu >> 3) + kg) * 16 + 4 * ((nu >> 1) & 3);
   const int shift = 8 * (nu & 1);  // h = nu%2 picks the low or the high byte pairs
@@ -145,10 +154,11 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   // 16j + 8h + 2s' + e of the block, s' the strip's place in the block.  The
   // per-channel scales of those columns are fetched now (wave s < CS writes
   // strip s in the end).
-  const int res_col = 64 * (strip0 >> 2) + 2 * (strip0 & 3) + 32 * (kg & 1) + (kg >> 1) + 2 * wave;
+  const int res_strip = strip0 + wave;
+  const int res_col = 64 * (res_strip >> 2) + 2 * (res_strip & 3) + 32 * (kg & 1) + (kg >> 1);
   unsigned short chan[4] = {0, 0, 0, 0};
   if constexpr (!GROUP) {
-    if (wave < CS) {
+    if (wave < CS && res_strip < n_strips) {
 #pragma unroll
       for (int r = 0; r < 4; r++)
         chan[r] = __builtin_amdgcn_raw_buffer_load_b16(
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
 
   const DequantConsts dc;
 
-  i4 bq[DEPTH][2];
+  i4 bq[DEPTH][NL];
   unsigned short sq[DEPTH][NSC > 0 ? NSC * CS : 1];
   i4 aq[DEPTH][Sh::kALoads];
 
@@ -190,8 +200,9 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
     // the weights last: what comes back first is small and near
     const int b_chunk = valid ? c * (KC * 2) * b_row : kStripOob;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
-      bq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rB, b_lane[i] + b_chunk, 0, 2);
+    for (int i = 0; i < NL; i++)
+      bq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(
+          rB, b_mine[i] ? b_lane[i] + b_chunk : kStripOob, 0, 2);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -208,13 +219,16 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
     const h2 mul = {(half_t)0.0625f, (half_t)0.0625f};
     const h2 add = {(half_t)-72.f, (half_t)-72.f};
     // Each of the chunk's two weight loads holds half its k steps and is used
-    // as it lands: registers -> LDS as fetched ([row][strip][Marlin lane]),
-    // then all operands of the half back from LDS before the first of them is
-    // used (read one k step at a time, every step would wait out a trip to LDS).
+    // as it lands (of three loads the first two hold the first half): registers
+    // -> LDS as fetched ([row][strip][Marlin lane]), then all operands of the
+    // half back from LDS before the first of them is used (read one k step at
+    // a time, every step would wait out a trip to LDS).
     constexpr int KH = KC / 2;
 #pragma unroll
     for (int half = 0; half < 2; half++) {
-      *(i4*)(stage + Sh::kWeightBase + (64 * half + lane) * 16) = bq[slot][half];
+#pragma unroll
+      for (int i = (half == 0 ? 0 : NL - 1); i < (half == 0 ? NL - 1 : NL); i++)
+        *(i4*)(stage + Sh::kWeightBase + (64 * i + lane) * 16) = bq[slot][i];
       i4 av[KH];
       int wv[KH][CS][2];
 #pragma unroll
@@ -273,7 +287,7 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
 #pragma unroll
   for (int s = 0; s < CS; s++) red[(wave * CS + s) * 64 + lane] = acc[s][0] + acc[s][1];
   __syncthreads();
-  if (wave < CS) {
+  if (wave < CS && res_strip < n_strips) {
     const int s = wave;
     f4 v = red[s * 64 + lane];
 #pragma unroll
@@ -311,14 +325,17 @@ static int configure_strip_width() {
 }
 
 int configure_strip_kernels() {
-  return (configure_strip_width<1>() | configure_strip_width<2>() | configure_strip_width<4>()) ? 3
-                                                                                                 : 0;
+  return (configure_strip_width<1>() | configure_strip_width<2>() | configure_strip_width<3>() |
+          configure_strip_width<4>())
+             ? 3
+             : 0;
 }
 
 template <int CS, int MR, bool GROUP>
 static int launch_strip_variant(const GemmArgs& a, hipStream_t stream) {
   constexpr int lds = StripShape<CS, MR>::kBytes;
-  const dim3 grid(a.N / (16 * CS) * (a.row_parts > 1 ? a.row_parts : 1)), block(64 * kStripWaves);
+  const dim3 grid(ceil_div(a.N / 16, CS) * (a.row_parts > 1 ? a.row_parts : 1)),
+      block(64 * kStripWaves);
   GemmArgs b = a;
   b.gpb = (int)grid.x;
   // Chunks in flight per wave: one where a wave has two at most, else two.
@@ -343,15 +360,19 @@ static int launch_strip_rows(const GemmArgs& a, hipStream_t stream) {
   return launch_strip_variant<CS, 16, GROUP>(a, stream);
 }
 
-// strips: 16-column strips per workgroup (1, 2 or 4; N a multiple of 16*strips)
+// strips: 16-column strips per workgroup (1, 2 or 4 with N a multiple of
+// 16*strips, or 3 with any N)
 int launch_strip(const GemmArgs& a, bool group, int strips, hipStream_t stream) {
   const int parts = a.row_parts > 1 ? a.row_parts : 1;
-  if (a.M > 16 * parts || a.M > kStripMaxRows || a.N % (16 * strips) != 0) return 2;
+  if (a.M > 16 * parts || a.M > kStripMaxRows || (strips != 3 && a.N % (16 * strips) != 0))
+    return 2;
   switch (strips * 2 + (group ? 1 : 0)) {
     case 2: return launch_strip_rows<1, false>(a, stream);
     case 3: return launch_strip_rows<1, true>(a, stream);
     case 4: return launch_strip_rows<2, false>(a, stream);
     case 5: return launch_strip_rows<2, true>(a, stream);
+    case 6: return launch_strip_rows<3, false>(a, stream);
+    case 7: return launch_strip_rows<3, true>(a, stream);
     case 8: return launch_strip_rows<4, false>(a, stream);
     case 9: return launch_strip_rows<4, true>(a, stream);
   }

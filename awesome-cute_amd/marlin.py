@@ -279,7 +279,7 @@ def force_kernel(which):
 
 
 def force_strips(strips):
-    """16-column strips per workgroup of the column-strip kernel (1, 2 or 4); 0 = choose by
+    """16-column strips per workgroup of the column-strip kernel (1 to 4); 0 = choose by
     cost (calling thread only)."""
     _lib.marlin_amd_force_strips(int(strips))
 

@@ -80,8 +80,9 @@ void marlin_amd_force_kernel(int which);
 
 /*
  * 16-column strips per workgroup of the column-strip kernel, for the calling
- * thread: 0 = choose by cost (default), or 1, 2, 4 (halved until prob_n is a
- * multiple of 16 x strips).  No reference counterpart; for tests and tools.
+ * thread: 0 = choose by cost (default), or 1 to 4 (2 and 4 only where prob_n
+ * is a multiple of 16 x strips, else 1; with 3 the last workgroup holds what
+ * is left).  No reference counterpart; for tests and tools.
  */
 void marlin_amd_force_strips(int strips);
 

@@ -256,10 +256,10 @@ def test_kernel_choice_by_cost(marlin):
     assert marlin.plan(1, 4096, 4096, 128, sms=64)[1]["kernel"] == 1  # a hint asks for the streaming split
     try:
         marlin.force_kernel(3)
-        for strips in (1, 2, 4):
+        for strips in (1, 2, 3, 4):
             marlin.force_strips(strips)
             rc, p = marlin.plan(16, 28672, 8192, 128)
-            assert (p["kernel"], p["strips"], p["grid"]) == (3, strips, 28672 // (16 * strips))
+            assert (p["kernel"], p["strips"], p["grid"]) == (3, strips, -(-28672 // (16 * strips)))
         marlin.force_strips(4)
         rc, p = marlin.plan(16, 128 * 3, 512, 128, 128, 128)  # 24 strips
         assert (p["kernel"], p["strips"]) == (3, 4) and p["grid"] == 6

@@ -3,7 +3,7 @@ dozen shapes from the decode to the prefill regime, the planned launch must not
 be more than 10 % slower than the best of the forced alternatives -- the
 streaming kernel, the prefill kernel on 64-row tiles and on 128-row tiles, each
 with the slice count its cost model picks, and for at most 1024 rows the
-column-strip kernel with 1, 2 and 4 strips per workgroup (for at most 16 rows
+column-strip kernel with 1 to 4 strips per workgroup (for at most 16 rows
 instead of the prefill kernel).  The planner is a fitted cost model;
 this test is what fails when a kernel change shifts the costs under it.  (The
 dispatch rules it replaces: reference marlin_cute_kernel.cu:39-49.)
@@ -87,7 +87,7 @@ def _measure(torch, marlin, m, n, k):
         marlin.force_kernel(1)
         times["streaming"] = _us_per_call(torch, call, 40)
         if m <= 1024:
-            for strips in (1, 2, 4):
+            for strips in (1, 2, 3, 4):
                 marlin.force_kernel(3)
                 marlin.force_strips(strips)
                 times[f"column strips, {strips} per workgroup"] = _us_per_call(torch, call, 40)
