@@ -439,15 +439,18 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
 // 1, 2 and 4 where they divide n's strips, and for up to 16 rows of 3, which
 // leaves the last workgroup with fewer (N = 11008, K = 4096, 230 workgroups
 // of three strips against 172 of four: M = 16 9.2 against 9.3 us, M = 8 8.2 /
-// 8.5, M = 1 7.5 / 7.7 with one strip; N = 5120, K = 5120: 10.3 against 8.4
-// with two)
+// 8.5, M = 1 7.5 / 7.7 with one strip; K = 8192: M = 1 12.3 against 13.6, M =
+// 4 11.7 / 13.6, M = 16 14.4 / 15.2; N = 5120, K = 5120: 10.3 against 8.4 with
+// two)
 // (0 where the planner's own rules leave none; a forced launch takes any)
 int strips_per_workgroup(int m, int n, int k, const PlanCtx& cx) {
   const bool forced = cx.force.kernel == 3 || cx.force.strips != 0;
   int best = 0;
   double best_cost = 0.0;
   for (int cs = 1; cs <= 4; cs++) {
-    if (cs == 3 ? (m > 16 && !forced) : n % (16 * cs) != 0) continue;
+    // (three strips: not over k ranges of a chunk or two per wave, where their
+    // three loads per chunk cost 8 % against two or four strips)
+    if (cs == 3 ? ((m > 16 || k < 1024) && !forced) : n % (16 * cs) != 0) continue;
     // Rows in parts: at most two workgroups per compute unit (with three and
     // more the streaming kernel was 1.1 to 1.6 times faster wherever the fits,
     // its own 20 to 40 % high over short k ranges, promised otherwise: 48 rows
