@@ -526,7 +526,7 @@ STRIP_SHAPES = [
 @pytest.mark.parametrize("strips", [1, 2, 3, 4])
 @pytest.mark.parametrize("m,n,k,g", STRIP_SHAPES)
 def test_column_strip_kernel(env, strips, m, n, k, g):
-    """The kernel whose workgroups own 16, 32 or 64 columns (and 16 rows) over
+    """The kernel whose workgroups own 16, 32, 48 or 64 columns (and 16 rows) over
     the whole k range and exchange nothing: every strip width on every shape,
     C overwritten everywhere (it starts at 9)."""
     torch, marlin = env
