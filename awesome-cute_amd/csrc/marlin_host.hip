@@ -308,7 +308,8 @@ double halves_gain(int rows, int wpt, int gpb) {
 // rows takes 11.3 + 0.28 per granule of the longest workgroup (N=K=4096: 8
 // granules, 12.9; N=8192, K=4096: 16, 15.5; N=4096, K=11008: 22, 18.0;
 // N=11008, K=4096 or 8192^2: 32, 18.5-20; N=28672, K=8192: 128, 46), fewer
-// rows a share of that, up to 16 rows 5.1 + 0.16 per granule; every launch
+// rows a share of that, up to 16 rows 4.9 + 0.17 per granule (1.4 less where
+// no tile is shared: N=28672, K=8192, 128 granules, 23 us); every launch
 // after the first waits a microsecond for the one before (65 rows at N=4096,
 // K=11008: 18.0 + 9.0 alone, 27.0 in a row).
 double stream_cost(int m, int n, int k, int cus) {
@@ -320,8 +321,11 @@ double stream_cost(int m, int n, int k, int cus) {
     t += full * (tail > 48 ? 1.0 : tail > 32 ? 0.9 : 0.65);
   } else if (tail > 0) {
     const StreamSplit s1 = choose_stream_split(1, n, k, cus);
-    t += 5.1 + 0.16 * s1.gpb + (s1.straddle ? 3.5 : 0.0) +
-         sharer_cost(s1.wpt > 0 ? s1.wpt : ceil_div(k / kGranuleK, s1.gpb));
+    // (refitted over M = 1, 4, 8, 16 on N = 256...28672, K = 512...11008, 6 %
+    // rms: a workgroup that shares its tiles with no other exchanges nothing)
+    const int sharers = s1.wpt > 0 ? s1.wpt : ceil_div(k / kGranuleK, s1.gpb);
+    t += 4.94 + 0.167 * s1.gpb + (tail > 8 ? 0.23 : 0.0) + (s1.straddle ? 3.5 : 0.0) +
+         (sharers == 1 && !s1.straddle ? -1.39 : sharer_cost(sharers));
   }
   return t + 1.0 * (ceil_div(m, kStreamMaxRows) - 1);
 }
@@ -415,6 +419,11 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
 // 256, K = 512 3.8.
 double strip_cost(int m, int n, int k, int cs, int cus) {
   const double by_memory = 0.5 * k * n / 4.8e6;
+  // a wave's chunk is 256 / cs k-values (128 with three strips): a k range of
+  // fewer than eight chunks leaves waves idle (K = 1024: one strip 0.2 to 0.3
+  // us behind two at every N from 8 rows on; fewer rows are no slower for it)
+  const int chunks = ceil_div(k, cs == 3 ? 128 : 256 / cs);
+  const double idle = m >= 8 && chunks < 8 ? 0.7 * (1.0 - chunks / 8.0) : 0.0;
   if (m > 16) {
     // rows in parts of 16, a workgroup each: fitted to 17...128 rows over N =
     // 256...28672, K = 512...11008 (8 % rms where the strips are within 1.6
@@ -423,16 +432,22 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
     const int rounds = ceil_div(wgs, cus);
     const double per_wg = 1.27 + 8.0 * cs * k / 32.7e3 + 32.0 * k / 67.8e3;
     const double by_cu = rounds * per_wg * (1.0 - 0.24 * (1.0 - 1.0 / rounds));
-    return 1.8 + (by_cu > by_memory ? by_cu : by_memory);
+    return 1.8 + (by_cu > by_memory ? by_cu : by_memory) + idle;
   }
   const int wgs = ceil_div(n / 16, cs);
   const int per_cu = ceil_div(wgs, cus);
-  const double by_cu = per_cu * 8.0 * cs * k / 23e3;
+  // (up to 8 rows the group scales go to the sums, not to the weights: fitted
+  // on its own over M = 1, 4, 8, 7 % rms)
+  const bool few = m <= 8;
+  const double by_cu = per_cu * 8.0 * cs * k / (few ? 28.0e3 : 23e3);
+  // (memory: 5.85 TB/s while every round of workgroups fills the compute units)
+  const double by_mem = 0.5 * k * n / (few ? 5.85e6 * (wgs > cus ? (double)wgs / (per_cu * cus) : 1.0) : 4.8e6);
   // (with 172 of 256 compute units reading 16 rows the rows came in a third
   // sooner than this: N = 11008, K = 4096 with four strips)
-  const double rows = per_cu * 2.0 * m * k / 87e3 * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
+  const double rows = per_cu * 2.0 * m * k / (few ? 72.5e3 : 87e3) * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
   // (a little of by_cu always: it decides between widths that memory bounds alike)
-  return 2.7 + (by_cu > by_memory ? by_cu : by_memory) + rows + 0.3 * (per_cu - 1) + 0.02 * by_cu;
+  return (few ? 2.88 : 2.7) + (by_cu > by_mem ? by_cu : by_mem) + rows + (few ? 0.43 : 0.3) * (per_cu - 1) +
+         0.02 * by_cu + idle;
 }
 
 // 16-column strips per workgroup of the column-strip kernel: the cheapest of

@@ -82,6 +82,12 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   constexpr int KC = Sh::kSteps;
   constexpr int NL = Sh::kLoads;
   constexpr int NSC = GROUP ? (CS == 1 ? 2 : 1) : 0;  // scale rows a chunk touches
+  // Group scales, up to 8 rows: applied to the sums of a group instead of to
+  // its weights (below).  With 16 rows staged the two forms are within 1.5 %
+  // of each other either way (M = 16: N = 11008, K = 4096 9.3 us against 9.2,
+  // N = K = 4096 5.85 / 5.83, N = 8192, K = 2048 5.0 / 5.1) and the weights
+  // keep their scales.
+  constexpr bool kScaleSums = GROUP && MR <= 8;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   {
@@ -130,10 +136,13 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   }
   const int b_rd = (4 * (nu >> 3) + kg) * 16 + 4 * ((nu >> 1) & 3);
   const int shift = 8 * (nu & 1);  // h = nu%2 picks the low or the high byte pairs
-  // group scales: a group's row holds the column of lane nu of strip S at
+  // group scales: a group's row holds the column of slot nu of strip S at
   // position 16S + 8e + 2j + h = 16S + nu (the 64-column permutation of
-  // reference marlin.py:50-51 puts the 8 columns of a Marlin lane side by side)
-  const int s_lane = 2 * (16 * strip0 + nu);
+  // reference marlin.py:50-51 puts the 8 columns of a Marlin lane side by side).
+  // Applied to the weights, MFMA lane (kg, nu) needs the scale of slot nu;
+  // applied to the sums, result lane (row, kg) needs those of the slots 4 kg
+  // ... 4 kg + 3, four scales in 8 bytes.
+  const int s_lane = 2 * (16 * strip0 + (kScaleSums ? 4 * kg : nu));
   // activations: lane (row, piece) fetches 16 bytes (8 k-values)
   const int a_row = lane / Sh::kLanesPerRow;
   const int a_piece = lane % Sh::kLanesPerRow;
@@ -169,7 +178,7 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   const DequantConsts dc;
 
   i4 bq[DEPTH][NL];
-  unsigned short sq[DEPTH][NSC > 0 ? NSC * CS : 1];
+  i2 sq[DEPTH][NSC > 0 ? NSC * CS : 1];
   i4 aq[DEPTH][Sh::kALoads];
 
   // Request chunk c into ring slot `slot`.  The per-lane part of an address is
@@ -193,7 +202,10 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
       for (int g = 0; g < NSC; g++) {
 #pragma unroll
         for (int s = 0; s < CS; s++)
-          sq[slot][g * CS + s] = __builtin_amdgcn_raw_buffer_load_b16(rS, vs + 32 * s, 0, 0);
+          if constexpr (kScaleSums)
+            sq[slot][g * CS + s] = __builtin_amdgcn_raw_buffer_load_b64(rS, vs + 32 * s, 0, 0);
+          else
+            sq[slot][g * CS + s][0] = __builtin_amdgcn_raw_buffer_load_b16(rS, vs + 32 * s, 0, 0);
         vs += p.N * 2;
       }
     }
@@ -209,6 +221,20 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
   f4 acc[CS][2];
 #pragma unroll
   for (int s = 0; s < CS; s++) acc[s][0] = acc[s][1] = (f4){0.f, 0.f, 0.f, 0.f};
+
+  // Group scales applied to the sums of a group: its k steps are summed from
+  // zero (`part`) and the sums scaled (fp32) into the accumulators -- four
+  // multiply-adds per group and strip instead of four packed multiplies per k
+  // step (M = 1: N = K = 4096 4.31 -> 4.22 us, 8192 x 8192 8.6 -> 8.2, N =
+  // 11008, K = 4096 7.5 -> 6.95; M = 8, N = K = 4096 5.04 -> 4.91).  One strip
+  // has a group per half chunk, more strips have one per chunk or two.  A
+  // one-hot row still returns fp16((q - 8) s), with its one rounding; sums of
+  // several weights are rounded once instead of once per weight.  (Scaling the
+  // sums only after the next operands have been read from LDS, when the
+  // group's last MFMA has long finished, was no faster: 4.29, 8.2, 7.1.)
+  f4 part[CS];
+#pragma unroll
+  for (int s = 0; s < CS; s++) part[s] = (f4){0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](int slot) {
     // activations of the chunk: registers -> LDS, rows as they are
@@ -256,17 +282,33 @@ __global__ __launch_bounds__(64 * kStripWaves) void strip_kernel(GemmArgs p) {
           h2 ha = __builtin_elementwise_fma(as_h2((wa & dc.hi_mask) | dc.ex), mul, add);
           h2 lb = as_h2((wb & dc.lo_mask) | dc.ex) - sub;
           h2 hb = __builtin_elementwise_fma(as_h2((wb & dc.hi_mask) | dc.ex), mul, add);
-          if constexpr (GROUP) {
+          if constexpr (GROUP && !kScaleSums) {
             const int g = CS == 1 ? q / 4 : 0;
-            const half_t sc = __builtin_bit_cast(half_t, sq[slot][g * CS + s]);
+            const half_t sc = __builtin_bit_cast(half_t, (unsigned short)sq[slot][g * CS + s][0]);
             const h2 s2 = {sc, sc};
             la *= s2;
             ha *= s2;
             lb *= s2;
             hb *= s2;
           }
-          acc[s][q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(make_h8(la, ha, lb, hb), af,
-                                                                 acc[s][q & 1], 0, 0, 0);
+          if constexpr (kScaleSums) {
+            const bool first = CS == 1 ? u == 0 : q == 0;
+            const f4 from = first ? (f4){0.f, 0.f, 0.f, 0.f} : part[s];
+            part[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(make_h8(la, ha, lb, hb), af, from, 0, 0, 0);
+          } else {
+            acc[s][q & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(make_h8(la, ha, lb, hb), af,
+                                                                   acc[s][q & 1], 0, 0, 0);
+          }
+        }
+      }
+      // (a group ends with every half chunk of one strip, else with the chunk)
+      if (kScaleSums && (CS == 1 || half == 1)) {
+#pragma unroll
+        for (int s = 0; s < CS; s++) {
+          const h4 sc = __builtin_bit_cast(h4, sq[slot][(CS == 1 ? half : 0) * CS + s]);
+#pragma unroll
+          for (int r = 0; r < 4; r++)
+            acc[s][0][r] = __builtin_fmaf((float)sc[r], part[s][r], acc[s][0][r]);
         }
       }
     }

@@ -252,7 +252,7 @@ def test_kernel_choice_by_cost(marlin):
     rc, p = marlin.plan(64, 4096, 4096, 128)
     assert (p["kernel"], p["strips"], p["row_parts"], p["part_rows"], p["grid"]) == (3, 4, 4, 16, 256)
     rc, p = marlin.plan(100, 512, 1024, 128)
-    assert (p["kernel"], p["strips"], p["row_parts"], p["grid"], p["launches"]) == (3, 1, 7, 32 * 7, 1)
+    assert (p["kernel"], p["strips"], p["row_parts"], p["grid"], p["launches"]) == (3, 2, 7, 16 * 7, 1)
     assert marlin.plan(1, 4096, 4096, 128, sms=64)[1]["kernel"] == 1  # a hint asks for the streaming split
     try:
         marlin.force_kernel(3)
