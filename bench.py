@@ -65,8 +65,8 @@ M_SWEEP = ["m32", "m64", "m128", "m256", "m512", "m1024"]
 # it was measured on (kernel, grid): when the library plans the shape otherwise
 # the figure is stale and is reported as null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode": (("strips", 256), int((4297.0 * 2.0 + 8.0) * 1024)),            # 8.81 MB, 1.02 x algorithmic
-    "batch16": (("strips", 256), int((4782.5 * 2.0 + 128.0) * 1024)),         # 9.93 MB, 1.11 x (the rows read by every workgroup)
+    "decode": (("strips", 256), int((4284.5 * 2.0 + 8.0) * 1024)),            # 8.78 MB, 1.01 x algorithmic
+    "batch16": (("strips", 256), int((4770.0 * 2.0 + 128.0) * 1024)),         # 9.90 MB, 1.11 x (the rows read by every workgroup)
     "prefill": (("prefill", 256), int((33941.5 * 2.0 + 16389.5) * 1024)),     # 86.3 MB, 2.04 x (A and B read by 16 tiles each)
     "mlp_up": (("strips", 230), int((11930.9 * 2.0 + 356.0) * 1024)),         # 24.8 MB, 1.04 x
     "mlp_down": (("stream", 256), int((13714.5 * 2.0 + 2185.0) * 1024)),      # 30.3 MB, 1.28 x
