@@ -611,6 +611,35 @@ def test_column_strip_kernel_closed_forms(env, strips, M):
         marlin.force_strips(0)
 
 
+@pytest.mark.parametrize("M", [1, 5, 8])
+@pytest.mark.parametrize("strips", [1, 2, 3, 4])
+def test_column_strip_kernel_scales_the_sums_of_a_group(env, strips, M):
+    """Up to 8 rows the column strips multiply the sum of a group by its scale
+    (fp32) instead of every weight (fp16): with small integer activations the
+    result is sum_g s_g * (integer), exact in fp32 up to the order of the adds,
+    so C is within one fp16 step of the exactly computed value -- nearer than
+    the per-weight rounding of the scaled weights would be."""
+    torch, marlin = env
+    N, K = 256, 1024
+    rng = np.random.default_rng(70 + strips + M)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float16)
+    q = rng.integers(0, 16, (K, N), dtype=np.uint8)
+    s = rng.uniform(0.001, 0.02, (K // 128, N)).astype(np.float16)
+    marlin.force_kernel(3)
+    marlin.force_strips(strips)
+    try:
+        C = gpu_gemm(env, A, O.pack_weights(q), O.pack_scales(s, True), N).astype(np.float64)
+    finally:
+        marlin.force_kernel(0)
+        marlin.force_strips(0)
+    want = np.zeros((M, N))
+    for g in range(K // 128):
+        rows = slice(128 * g, 128 * g + 128)
+        want += s[g].astype(np.float64) * (A[:, rows].astype(np.int64) @ (q[rows].astype(np.int64) - 8))
+    step = np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -10  # one step of fp16 at |want|
+    assert (np.abs(C - want) <= step).all(), np.abs((C - want) / step).max()
+
+
 def test_few_rows_through_either_kernel_agree_with_the_oracle(env):
     """The shapes the planner gives to the column strips, through the streaming
     kernel as well: both inside the tolerance, on the same inputs."""
