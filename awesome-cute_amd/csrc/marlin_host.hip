@@ -418,7 +418,6 @@ bool prefer_prefill(int m, int n, int k, const PlanCtx& cx) {
 // 512 3.4, 2048 x 2048 6.8; M = 512: N = 256, K = 1024 3.7; M = 1024: N =
 // 256, K = 512 3.8.
 double strip_cost(int m, int n, int k, int cs, int cus) {
-  const double by_memory = 0.5 * k * n / 4.8e6;
   // a wave's chunk is 256 / cs k-values (128 with three strips): a k range of
   // fewer than eight chunks leaves waves idle (K = 1024: one strip 0.2 to 0.3
   // us behind two at every N from 8 rows on; fewer rows are no slower for it)
@@ -432,22 +431,27 @@ double strip_cost(int m, int n, int k, int cs, int cus) {
     const int rounds = ceil_div(wgs, cus);
     const double per_wg = 1.27 + 8.0 * cs * k / 32.7e3 + 32.0 * k / 67.8e3;
     const double by_cu = rounds * per_wg * (1.0 - 0.24 * (1.0 - 1.0 / rounds));
+    const double by_memory = 0.5 * k * n / 4.8e6;
     return 1.8 + (by_cu > by_memory ? by_cu : by_memory) + idle;
   }
+  // Up to 8 rows the group scales go to the sums, not to the weights, and the
+  // constants are fitted on their own (M = 1, 4, 8: 7 % rms): the launch, the
+  // rate a compute unit unpacks at, the rate it reads rows at, a queued
+  // workgroup, and memory -- 5.85 TB/s while every round of workgroups fills
+  // the compute units.
+  const bool few = m <= 8;
   const int wgs = ceil_div(n / 16, cs);
   const int per_cu = ceil_div(wgs, cus);
-  // (up to 8 rows the group scales go to the sums, not to the weights: fitted
-  // on its own over M = 1, 4, 8, 7 % rms)
-  const bool few = m <= 8;
+  const double last_round = wgs > cus ? (double)wgs / (per_cu * cus) : 1.0;
   const double by_cu = per_cu * 8.0 * cs * k / (few ? 28.0e3 : 23e3);
-  // (memory: 5.85 TB/s while every round of workgroups fills the compute units)
-  const double by_mem = 0.5 * k * n / (few ? 5.85e6 * (wgs > cus ? (double)wgs / (per_cu * cus) : 1.0) : 4.8e6);
+  const double by_memory = 0.5 * k * n / (few ? 5.85e6 * last_round : 4.8e6);
   // (with 172 of 256 compute units reading 16 rows the rows came in a third
   // sooner than this: N = 11008, K = 4096 with four strips)
-  const double rows = per_cu * 2.0 * m * k / (few ? 72.5e3 : 87e3) * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
+  const double rows =
+      per_cu * 2.0 * m * k / (few ? 72.5e3 : 87e3) * (wgs < cus ? (0.5 + 0.5 * wgs / cus) : 1.0);
   // (a little of by_cu always: it decides between widths that memory bounds alike)
-  return (few ? 2.88 : 2.7) + (by_cu > by_mem ? by_cu : by_mem) + rows + (few ? 0.43 : 0.3) * (per_cu - 1) +
-         0.02 * by_cu + idle;
+  return (few ? 2.88 : 2.7) + (by_cu > by_memory ? by_cu : by_memory) + rows +
+         (few ? 0.43 : 0.3) * (per_cu - 1) + 0.02 * by_cu + idle;
 }
 
 // 16-column strips per workgroup of the column-strip kernel: the cheapest of
