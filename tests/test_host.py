@@ -322,6 +322,39 @@ def test_plan_costs_are_what_the_choice_compares(marlin):
         assert marlin.plan(m, n, k, 128)[1]["kernel"] == want, (m, n, k, c)
 
 
+def test_planned_column_strips_obey_the_planner_s_rules(marlin):
+    """Over random shapes: a planned column-strip launch has strip sets x 16-row
+    parts workgroups in one launch without scratch; more than 16 rows only while
+    the parts fill 256 compute units at most twice; three strips per workgroup
+    only up to 16 rows and from K = 1024 on; two and four only where they divide
+    N's strips; nothing beyond 1024 rows or with an `sms` hint."""
+    rng = np.random.default_rng(5)
+    seen = 0
+    for _ in range(3000):
+        m = int(rng.choice([1, 2, 5, 8, 9, 16, 17, 33, 64, 100, 256, 700, 1024, 1025, 3000]))
+        n = 256 * int(rng.integers(1, 120)) if m > 16 or rng.random() < 0.5 else 128 * int(rng.integers(1, 240))
+        k = 128 * int(rng.integers(1, 100))
+        sms = int(rng.choice([-1, -1, -1, 64]))
+        rc, p = marlin.plan(m, n, k, 128, sms=sms)
+        assert rc == 0, (m, n, k)
+        if p["kernel"] != 3:
+            assert p["strips"] == 0
+            continue
+        seen += 1
+        cs, parts = p["strips"], -(-m // 16)
+        assert sms < 0 and m <= 1024 and cs in (1, 2, 3, 4)
+        assert p["row_parts"] == parts and p["part_rows"] == (16 if m > 16 else 0)
+        assert p["grid"] == -(-(n // 16) // cs) * parts
+        assert p["launches"] == 1 and p["partial_kib"] == 0
+        if m > 16:
+            assert p["grid"] <= 2 * 256, (m, n, k, p)
+        if cs == 3:
+            assert m <= 16 and k >= 1024
+        else:
+            assert n % (16 * cs) == 0
+    assert seen > 300
+
+
 def test_plan_picks_kernels(marlin):
     assert marlin.plan(1, 4096, 4096, 128)[1]["kernel"] == 3
     assert marlin.plan(32, 28672, 8192, 128)[1]["kernel"] == 1
