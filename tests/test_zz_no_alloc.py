@@ -106,6 +106,13 @@ def test_static_entry_through_column_strips(env):
     assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
     r = O.compare(c_static, O.gemm(A, B, sp, 4096, 128))
     assert r.max_abs_err <= TOL * r.max_abs_ref
+    # ... and for more rows in parts of 16 (here seven, the last with four rows)
+    p = marlin.plan(100, 1024, 1024, -1)[1]
+    assert (p["kernel"], p["row_parts"], p["partial_kib"]) == (3, 7, 0)
+    (A, B, sp), c_static, c_pool = both(env, 100, 1024, 1024, -1, seed=78)
+    assert np.array_equal(c_static.view(np.uint16), c_pool.view(np.uint16))
+    r = O.compare(c_static, O.gemm(A, B, sp, 1024, -1))
+    assert r.max_abs_err <= TOL * r.max_abs_ref
 
 
 def test_rejects_what_does_not_fit(env):
